@@ -1,0 +1,197 @@
+/* tmx: MI355X (gfx950) decode-step kernels for an int4 group-quantised QLoRA
+ * policy behind tunix's Sampler -- C ABI.
+ *
+ * The reference (bigdatamark/tunix) has no FFI for this path: its decode step is
+ * XLA-compiled JAX.  Each entry point below names the reference arithmetic it
+ * replaces (path:line relative to the reference tree).  The same functions are
+ * what an XLA custom-call handler registered through jax.ffi would forward to.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - `stream` is a hipStream_t passed as void*; entry points only enqueue work
+ *     on it: they never allocate, free or synchronise;
+ *   - bf16 tensors are raw 16-bit patterns, row-major, innermost index last;
+ *   - return value: TMX_OK or a negative TMX_ERR_* code, nothing is launched
+ *     when an argument check fails.
+ *
+ * Packed int4 tile format ("q4t") of a logical weight W[K, N] (K % 64 == 0,
+ * N % 32 == 0), nibble u = q + 8 with q in [-8, 7]:
+ *   tile (nb, kb) = rows [64 kb, 64 kb + 64) x columns [32 nb, 32 nb + 32) is the
+ *   1024 bytes at byte offset (nb * (K / 64) + kb) * 1024; inside it lane
+ *   l = 32 h + (n % 32) owns the 16 bytes at l * 16 = four little-endian 32-bit
+ *   words t = 0..3; nibble i (bits 4i..4i+3) of word t is the element
+ *   k = 64 kb + 16 t + 8 h + 2 (i % 4) + (i / 4).
+ *   Scales: bf16 [N / 32][K / G][32], G % 64 == 0.
+ */
+#ifndef TMX_H_
+#define TMX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TMX_OK 0
+#define TMX_ERR_ARG (-1)         /* null pointer / inconsistent optional arguments */
+#define TMX_ERR_SHAPE (-2)       /* a dimension violates the kernel's tiling rules */
+#define TMX_ERR_LAUNCH (-3)      /* the HIP runtime refused the launch */
+#define TMX_ERR_UNSUPPORTED (-4) /* valid request outside what is implemented */
+
+#define TMX_FAMILY_LLAMA3 0
+#define TMX_FAMILY_QWEN3 1
+
+#define TMX_SAMPLE_GREEDY 0
+#define TMX_SAMPLE_TOP_P 1
+
+const char* tmx_status_string(int status);
+int tmx_abi_version(void);
+
+/* w_out[K, N] bf16 = bf16(q) * scale evaluated in bf16, bit-exact.
+ * Replaces qwix's dequantise step behind tunix/cli/utils/model.py:31-77
+ * (weight_qtype / tile_size of the LoraProvider). */
+int tmx_int4_dequant(void* stream, const void* qweight, const void* scales, void* w_out, int K, int N,
+                     int G);
+
+/* y[M, N] = bf16(x[M, K] . dequant(qweight)) (+ LoRA delta) (+ residual).
+ * Replaces the qwix-wrapped Einsum / nnx.Linear call: tunix/models/llama3/model.py:216-218,
+ * :489-496; tunix/models/qwen3/model.py:389-393, :1199-1208.
+ *   lora_a_t : A transposed and zero-padded, bf16 [r_pad, K], r_pad % 32 == 0 (NULL: no LoRA)
+ *   lora_b   : bf16 [r, N];  t_ws: bf16 [M, r_pad] workspace receiving x . A
+ *   residual : bf16 [M, N] or NULL; added after the LoRA delta, in bf16 */
+int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const void* scales,
+                     const void* lora_a_t, const void* lora_b, const void* residual, void* y, void* t_ws,
+                     int M, int K, int N, int G, int r, int r_pad, float lora_scale);
+
+/* ---- row-wise kernels between the matrix products ------------------------- */
+
+/* y[M, D] = RMSNorm(x) * w.  TMX_FAMILY_LLAMA3: bf16(bf16(w * x) / rms)
+ * (tunix/models/llama3/model.py:290-297); TMX_FAMILY_QWEN3: bf16(w * (x / rms))
+ * in f32 (tunix/models/qwen3/model.py:478-484). */
+int tmx_rmsnorm(void* stream, const void* x, const void* w, void* y, int M, int D, float eps, int family);
+
+/* h = bf16(bf16(y + lora_delta) + residual) -> x_out;  xn_out = RMSNorm(h) * norm_w.
+ * lora_delta[m, n] = bf16(bf16(sum_r t[m, r] lora_b[r, n]) * lora_scale); t, residual,
+ * x_out, norm_w may be NULL.  Residual wiring of tunix/models/llama3/model.py:546-564,
+ * tunix/models/qwen3/model.py:1268-1289. */
+int tmx_lora_residual_rmsnorm(void* stream, const void* y, const void* t, int ldt, const void* lora_b,
+                              int r, float lora_scale, const void* residual, void* x_out,
+                              const void* norm_w, void* xn_out, int M, int D, float eps, int family);
+
+/* qkv[B, (N + 2 Kh) H] (+ LoRA deltas, t = x.A_q | x.A_k | x.A_v) -> optional per-head
+ * RMSNorm (Qwen3 q_norm / k_norm), RoPE at positions[b, *step], q_out[B, N H] and the
+ * K / V rows of cache slot *step % C.  tunix/models/llama3/model.py:249-270, :348-377;
+ * tunix/models/qwen3/model.py:432-453, :559-597. */
+int tmx_rope_kv_write(void* stream, const void* qkv, const void* t, int ldt, const void* lora_b, int r,
+                      float lora_scale, const void* q_norm_w, const void* k_norm_w,
+                      const int32_t* positions, const int32_t* step, int buf_len, void* q_out,
+                      void* kcache, void* vcache, int B, int N, int Kh, int H, int C, float theta,
+                      float eps, int family);
+
+/* act[M, F] = bf16(silu(gate) * up), gate_up[M, 2F] = gate columns then up columns
+ * (+ LoRA deltas, t = x.A_gate | x.A_up).  tunix/models/llama3/model.py:489-496. */
+int tmx_swiglu(void* stream, const void* gate_up, const void* t, int ldt, const void* lora_b, int r,
+               float lora_scale, void* act, int M, int F);
+
+/* ---- GQA decode attention -------------------------------------------------- */
+
+/* out[B, N H] = softmax(q . K^T / sqrt(H) over positions j <= *step with
+ * input_mask[b, j]) . V, caches bf16 [B, C, Kh, H].  tunix/models/llama3/model.py:379-396,
+ * tunix/models/qwen3/model.py:776-793 with the mask of tunix/generate/utils.py:35-59.
+ * workspace: tmx_gqa_decode_workspace_bytes() bytes (may be 0 -> NULL allowed). */
+size_t tmx_gqa_decode_workspace_bytes(int B, int N, int Kh, int H, int C);
+int tmx_gqa_decode_attention(void* stream, const void* q, const void* kcache, const void* vcache,
+                             const uint8_t* input_mask, const int32_t* step, int buf_len, void* out,
+                             void* workspace, int B, int N, int Kh, int H, int C);
+
+/* ---- final projection + log-softmax + token selection ---------------------- */
+
+/* logits = bf16(x[M, D] . head_w[V, D]^T) as f32; forbidden ids -> -inf; mode
+ * TMX_SAMPLE_GREEDY: token = argmax (first index on ties), logprob =
+ * log_softmax(logits)[token]; TMX_SAMPLE_TOP_P (top_p >= 1, no top_k): z = logits /
+ * temperature, token = argmax(z + gumbel(threefry(fold_in(seed, *step)))), logprob =
+ * log_softmax(z)[token].  Writes token_buffer[m, *step + 1], logprobs[m, *step + 1]
+ * (if not NULL), done[m] |= token in eos.  tunix/generate/sampler.py:112-168, :520-599;
+ * tunix/models/llama3/model.py:688-697.  logits_out: optional f32 [M, V]. */
+size_t tmx_head_sample_workspace_bytes(int M, int V);
+int tmx_head_sample(void* stream, const void* x, const void* head_w, int M, int D, int V, int mode,
+                    float temperature, uint32_t seed_hi, uint32_t seed_lo, const int32_t* step,
+                    const int32_t* forbidden, int n_forbidden, const int32_t* eos, int n_eos,
+                    int32_t* token_buffer, float* logprobs, uint8_t* done, int buf_len,
+                    float* logits_out, void* workspace);
+
+/* ---- whole decode steps ------------------------------------------------------ */
+
+#define TMX_MAX_RPAD 128 /* widest padded LoRA projection (sum of fused ranks, rounded up to 32) */
+
+typedef struct {
+  const void* qweight;  /* q4t tiles of the (column-fused) weight [K, N] */
+  const void* scales;   /* bf16 [N/32][K/G][32] */
+  const void* lora_a_t; /* bf16 [r_pad, K]: fused A matrices side by side, transposed; NULL = no LoRA */
+  const void* lora_b;   /* bf16 [rank, N]: B matrices side by side */
+  int K, N, G, rank, r_pad;
+  float lora_scale;     /* alpha / rank */
+} tmx_qlinear_desc;
+
+typedef struct {
+  const void* norm1_w;  /* input_layernorm.w [D] bf16 */
+  const void* norm2_w;  /* post_attention_layernorm.w [D] */
+  const void* q_norm_w; /* Qwen3 q_norm.w [H] or NULL */
+  const void* k_norm_w;
+  tmx_qlinear_desc qkv;     /* columns: q (N H) | k (Kh H) | v (Kh H) */
+  tmx_qlinear_desc o;       /* [N H, D] */
+  tmx_qlinear_desc gate_up; /* columns: gate (F) | up (F) */
+  tmx_qlinear_desc down;    /* [F, D] */
+} tmx_layer_desc;
+
+typedef struct {
+  int family; /* TMX_FAMILY_* */
+  int num_layers, vocab_size, embed_dim, hidden_dim, num_heads, num_kv_heads, head_dim;
+  int num_experts, experts_per_tok;
+  float rope_theta; /* ignored for TMX_FAMILY_LLAMA3: the reference's Llama3 attention never
+                       forwards config.rope_theta, so 1e6 is used (llama3/model.py:356-365) */
+  float norm_eps;
+  const void* embed;        /* bf16 [V, D] */
+  const void* final_norm_w; /* bf16 [D] */
+  const void* head;         /* bf16 [V, D]: the embedding table when tied, else lm_head^T */
+  const tmx_layer_desc* layers; /* HOST array of num_layers entries */
+} tmx_model_desc;
+
+/* Mirrors _SamplingState (tunix/generate/sampler.py:53-109); all arrays on the device. */
+typedef struct {
+  int batch, buf_len, cache_size;
+  int32_t* token_buffer; /* [B, buf_len] */
+  int32_t* positions;    /* [B, buf_len] */
+  uint8_t* input_mask;   /* [B, buf_len] 1 = real token */
+  float* logprobs;       /* [B, buf_len] or NULL */
+  uint8_t* done;         /* [B] */
+  int32_t* step;         /* device scalar: decoding_step */
+  void* kv_cache;        /* bf16 [layers][2 (k, v)][B][C][Kh][H] */
+  int sampling_mode;     /* TMX_SAMPLE_* */
+  float temperature, top_p;
+  int top_k;
+  uint32_t seed_hi, seed_lo;
+  const int32_t* eos_ids;
+  int n_eos;
+  const int32_t* forbidden;
+  int n_forbidden;
+  float* logits_out;     /* optional f32 [B, V]: logits of the last executed step */
+  void* workspace;
+  size_t workspace_bytes;
+} tmx_decode_state;
+
+size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int cache_size);
+
+/* Enqueues n_steps iterations of the Sampler's decode loop body
+ * (tunix/generate/sampler.py:749-793): read token_buffer[:, *step], run the model with
+ * the KV cache, select the next token into column *step + 1, ++*step.  With sample == 0
+ * the head and token selection are skipped (cache fill: used to walk over prompt tokens).
+ * `model`, `state` and model->layers are HOST structures read during the call only. */
+int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
+                     int n_steps, int sample);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TMX_H_ */

@@ -1,0 +1,77 @@
+"""ctypes binding of libtmx.so (the C ABI declared in include/tmx.h).
+
+There is no CPU fallback: if the library is missing every operator raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'libtmx.so')
+
+_lib = None
+
+vp, ci, cf, cu32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_uint32
+
+# name -> argtypes (restype is int unless noted)
+SIGNATURES = {
+    'tmx_abi_version': [],
+    'tmx_int4_dequant': [vp, vp, vp, vp, ci, ci, ci],
+    'tmx_qlora_linear': [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
+    'tmx_rmsnorm': [vp, vp, vp, vp, ci, ci, cf, ci],
+    'tmx_lora_residual_rmsnorm': [vp, vp, vp, ci, vp, ci, cf, vp, vp, vp, vp, ci, ci, cf, ci],
+    'tmx_rope_kv_write': [vp, vp, vp, ci, vp, ci, cf, vp, vp, vp, vp, ci, vp, vp, vp, ci, ci, ci, ci, ci,
+                          cf, cf, ci],
+    'tmx_swiglu': [vp, vp, vp, ci, vp, ci, cf, vp, ci, ci],
+    'tmx_gqa_decode_attention': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci],
+    'tmx_head_sample': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
+                        vp, vp],
+    'tmx_decode_steps': [vp, vp, vp, ci, ci],
+}
+# entry points that return size_t
+SIZE_FUNCS = {
+    'tmx_gqa_decode_workspace_bytes': [ci, ci, ci, ci, ci],
+    'tmx_head_sample_workspace_bytes': [ci, ci],
+    'tmx_decode_workspace_bytes': [vp, ci, ci],
+}
+
+
+class TmxError(RuntimeError):
+  pass
+
+
+def lib():
+  """Loads the library once; raises if it has not been built."""
+  global _lib
+  if _lib is None:
+    if not os.path.exists(LIB_PATH):
+      raise TmxError(
+          f'{LIB_PATH} is missing: build it with `python -m tunix_amd.build` '
+          '(there is no CPU fallback for the decode path).')
+    l = ctypes.CDLL(LIB_PATH)
+    for name, args in SIGNATURES.items():
+      fn = getattr(l, name)
+      fn.argtypes = args
+      fn.restype = ci
+    for name, args in SIZE_FUNCS.items():
+      fn = getattr(l, name)
+      fn.argtypes = args
+      fn.restype = ctypes.c_size_t
+    l.tmx_status_string.argtypes = [ci]
+    l.tmx_status_string.restype = ctypes.c_char_p
+    _lib = l
+  return _lib
+
+
+def check(status, what):
+  if status != 0:
+    raise TmxError(f'{what}: {lib().tmx_status_string(status).decode()} (status {status})')
+
+
+def ptr(t):
+  """Device pointer of a torch tensor (None -> NULL)."""
+  return None if t is None else t.data_ptr()
+
+
+def stream():
+  import torch
+  return torch.cuda.current_stream().cuda_stream

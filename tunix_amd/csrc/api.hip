@@ -1,0 +1,15 @@
+// Status strings and ABI version of the C interface.
+#include "tmx_common.h"
+
+extern "C" const char* tmx_status_string(int status) {
+  switch (status) {
+    case TMX_OK: return "ok";
+    case TMX_ERR_ARG: return "invalid argument (null pointer or inconsistent optional arguments)";
+    case TMX_ERR_SHAPE: return "shape violates the kernel's tiling rules";
+    case TMX_ERR_LAUNCH: return "HIP launch failed";
+    case TMX_ERR_UNSUPPORTED: return "unsupported configuration";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int tmx_abi_version(void) { return 1; }

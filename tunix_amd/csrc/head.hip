@@ -1,0 +1,273 @@
+// Final projection to the vocabulary fused with log-softmax statistics and token
+// selection, so the [B, V] logits never travel through HBM.
+//
+// Replaces the tail of the model call and Sampler._sample:
+//   logits = bf16(x . head) -> f32      tunix/models/llama3/model.py:688-697, :244-246
+//                                       tunix/models/qwen3/model.py:1422-1442, :425-429
+//   forbidden ids -> -inf               tunix/generate/sampler.py:536-537
+//   greedy: argmax, first index on ties tunix/generate/sampler.py:158-168
+//   top_p mode with top_p >= 1, no top_k: z = logits / T, token = categorical(
+//     fold_in(seed, step), z), logprob = log_softmax(z)[token]
+//                                       tunix/generate/sampler.py:112-134, :562
+//   token / logprob scatter, done |= isin(token, eos)   tunix/generate/sampler.py:575-581
+//
+// categorical(key, z) = argmax(z + gumbel), gumbel from threefry2x32 bits over
+// the linear index b * V + v (jax's partitionable bit generation).
+//
+// Mapping: the head matrix [V, D] (bf16, the tied embedding table or the
+// transposed lm_head) is the A operand of v_mfma_f32_32x32x16_bf16, the hidden
+// states the B operand, so a lane's accumulator registers are 16 vocabulary rows
+// of ONE sequence: max / sum-exp / arg-best run down the registers without
+// cross-lane traffic.  Workgroup partials are merged by a second tiny kernel.
+#include "tmx_kernels.h"
+
+namespace tmx {
+
+__device__ __forceinline__ uint32_t rotl32(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
+
+__device__ __forceinline__ void threefry2x32(uint32_t k0, uint32_t k1, uint32_t c0, uint32_t c1,
+                                             uint32_t& o0, uint32_t& o1) {
+  const uint32_t ks[3] = {k0, k1, k0 ^ k1 ^ 0x1BD11BDAu};
+  uint32_t x0 = c0 + ks[0], x1 = c1 + ks[1];
+  const int rot[2][4] = {{13, 15, 26, 6}, {17, 29, 16, 24}};
+#pragma unroll
+  for (int g = 0; g < 5; ++g) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x0 += x1;
+      x1 = rotl32(x1, rot[g & 1][i]);
+      x1 ^= x0;
+    }
+    x0 += ks[(g + 1) % 3];
+    x1 += ks[(g + 2) % 3] + (uint32_t)(g + 1);
+  }
+  o0 = x0;
+  o1 = x1;
+}
+
+__device__ __forceinline__ float gumbel_from_bits(uint32_t bits) {
+  const float tiny = 1.17549435e-38f;
+  float f = __uint_as_float((bits >> 9) | 0x3F800000u) - 1.0f;
+  f = fmaxf(tiny, f + tiny);
+  return -logf(-logf(f));
+}
+
+struct Best {
+  float key;  // z + gumbel (or raw logit for greedy)
+  float z;
+  int idx;
+};
+__device__ __forceinline__ void best_merge(Best& a, const Best& b) {
+  if (b.key > a.key || (b.key == a.key && b.idx < a.idx)) a = b;
+}
+// (mx, se) <- merge with (mx2, se2): running max and sum of exp(z - max)
+__device__ __forceinline__ void lse_merge(float& mx, float& se, float mx2, float se2) {
+  const float mn = fmaxf(mx, mx2);
+  se = se * expf(mx - mn) + se2 * expf(mx2 - mn);
+  mx = mn;
+}
+
+
+constexpr float kNegBig = -3.0e38f;
+
+template <int MT>
+__global__ __launch_bounds__(256) void head_kernel(HeadArgs a) {
+  __shared__ float s_f[4][MT * 32][4];
+  __shared__ int s_i[4][MT * 32];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int h = lane >> 5, nl = lane & 31;
+  const int tile = blockIdx.x * 4 + wave;
+  const bool live = tile * 32 < a.V;
+  const int v0 = live ? tile * 32 : 0;
+
+  f32x16_t acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
+
+  const uint16_t* wrow = a.w + (size_t)(v0 + nl) * a.D + h * 32;
+  const uint16_t* xrow[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    int row = m * 32 + nl;
+    row = row < a.M ? row : a.M - 1;
+    xrow[m] = a.x + (size_t)row * a.D + h * 32;
+  }
+  if (live) {
+    for (int kb = 0; kb < a.D; kb += 64) {
+      bf16x8_t wf[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) wf[t] = *reinterpret_cast<const bf16x8_t*>(wrow + kb + t * 8);
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const bf16x8_t xf = *reinterpret_cast<const bf16x8_t*>(xrow[m] + kb + t * 8);
+          acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[t], xf, acc[m], 0, 0, 0);
+        }
+    }
+  }
+
+  // per-step key = fold_in(seed, step)
+  uint32_t key0 = 0, key1 = 0;
+  if (a.mode == TMX_SAMPLE_TOP_P) threefry2x32(a.k0, a.k1, 0u, (uint32_t)*a.step, key0, key1);
+
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int row = m * 32 + nl;
+    float mx = kNegBig, se = 0.f;
+    Best best = {-INFINITY, -INFINITY, 0x7FFFFFFF};
+    if (live && row < a.M) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int v = v0 + acc_row(r, lane);
+        float logit = rbf(acc[m][r]);
+        if (a.logits_out) a.logits_out[(size_t)row * a.V + v] = logit;
+        for (int f = 0; f < a.n_forbidden; ++f)
+          if (a.forbidden[f] == v) logit = -INFINITY;
+        float z = logit, key = logit;
+        if (a.mode == TMX_SAMPLE_TOP_P) {
+          z = logit / a.temperature;
+          uint32_t o0, o1;
+          threefry2x32(key0, key1, 0u, (uint32_t)row * (uint32_t)a.V + (uint32_t)v, o0, o1);
+          key = z + gumbel_from_bits(o0 ^ o1);
+        }
+        if (z > mx) {
+          se = se * expf(mx - z) + 1.f;
+          mx = z;
+        } else {
+          se += expf(z - mx);
+        }
+        Best c = {key, z, v};
+        best_merge(best, c);
+      }
+    }
+    // the other half-wave holds the other 16 vocabulary rows of the same sequence
+    {
+      const float mx2 = __shfl_xor(mx, 32, 64), se2 = __shfl_xor(se, 32, 64);
+      Best o = {__shfl_xor(best.key, 32, 64), __shfl_xor(best.z, 32, 64), __shfl_xor(best.idx, 32, 64)};
+      lse_merge(mx, se, mx2, se2);
+      best_merge(best, o);
+    }
+    if (h == 0) {
+      s_f[wave][row][0] = mx;
+      s_f[wave][row][1] = se;
+      s_f[wave][row][2] = best.key;
+      s_f[wave][row][3] = best.z;
+      s_i[wave][row] = best.idx;
+    }
+  }
+  __syncthreads();
+  for (int row = threadIdx.x; row < MT * 32; row += 256) {
+    if (row >= a.M) continue;
+    float mx = s_f[0][row][0], se = s_f[0][row][1];
+    Best best = {s_f[0][row][2], s_f[0][row][3], s_i[0][row]};
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      lse_merge(mx, se, s_f[w][row][0], s_f[w][row][1]);
+      Best o = {s_f[w][row][2], s_f[w][row][3], s_i[w][row]};
+      best_merge(best, o);
+    }
+    float* pf = a.part_f + ((size_t)row * a.nwg + blockIdx.x) * 4;
+    pf[0] = mx; pf[1] = se; pf[2] = best.key; pf[3] = best.z;
+    a.part_i[(size_t)row * a.nwg + blockIdx.x] = best.idx;
+  }
+}
+
+// One workgroup per sequence: merge the vocabulary-tile partials, emit the token
+// and its log-probability into column step + 1, update `done`.
+__global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
+  __shared__ float s_f[4][4];
+  __shared__ int s_i[4];
+  const int row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float mx = kNegBig, se = 0.f;
+  Best best = {-INFINITY, -INFINITY, 0x7FFFFFFF};
+  for (int i = threadIdx.x; i < a.nwg; i += 256) {
+    const float* pf = a.part_f + ((size_t)row * a.nwg + i) * 4;
+    lse_merge(mx, se, pf[0], pf[1]);
+    Best o = {pf[2], pf[3], a.part_i[(size_t)row * a.nwg + i]};
+    best_merge(best, o);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float mx2 = __shfl_xor(mx, off, 64), se2 = __shfl_xor(se, off, 64);
+    Best o = {__shfl_xor(best.key, off, 64), __shfl_xor(best.z, off, 64), __shfl_xor(best.idx, off, 64)};
+    lse_merge(mx, se, mx2, se2);
+    best_merge(best, o);
+  }
+  if (lane == 0) {
+    s_f[wave][0] = mx; s_f[wave][1] = se; s_f[wave][2] = best.key; s_f[wave][3] = best.z;
+    s_i[wave] = best.idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    mx = s_f[0][0]; se = s_f[0][1];
+    best = {s_f[0][2], s_f[0][3], s_i[0]};
+    for (int w = 1; w < 4; ++w) {
+      lse_merge(mx, se, s_f[w][0], s_f[w][1]);
+      Best o = {s_f[w][2], s_f[w][3], s_i[w]};
+      best_merge(best, o);
+    }
+    const int col = *a.step + 1;
+    const int tok = best.idx;
+    a.token_buffer[(size_t)row * a.buf_len + col] = tok;
+    if (a.logprobs) a.logprobs[(size_t)row * a.buf_len + col] = (best.z - mx) - logf(se);
+    bool hit = false;
+    for (int e = 0; e < a.n_eos; ++e) hit = hit || (a.eos[e] == tok);
+    if (hit) a.done[row] = 1;
+  }
+}
+
+int head_sample(hipStream_t st, HeadArgs a) {
+  if (a.V % 32 || a.D % 64 || a.M <= 0 || a.M > 128) return TMX_ERR_SHAPE;
+  a.nwg = (a.V + 127) / 128;
+  if (a.M <= 32) hipLaunchKernelGGL(head_kernel<1>, dim3(a.nwg), dim3(256), 0, st, a);
+  else if (a.M <= 64) hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(head_kernel<4>, dim3(a.nwg), dim3(256), 0, st, a);
+  int rc = check_launch();
+  if (rc != TMX_OK) return rc;
+  hipLaunchKernelGGL(head_finalize_kernel, dim3(a.M), dim3(256), 0, st, a);
+  return check_launch();
+}
+
+size_t head_partial_bytes(int M, int V) {
+  const size_t nwg = (V + 127) / 128;
+  return (size_t)M * nwg * 5 * sizeof(float);
+}
+
+}  // namespace tmx
+
+using namespace tmx;
+
+extern "C" size_t tmx_head_sample_workspace_bytes(int M, int V) { return head_partial_bytes(M, V); }
+
+extern "C" int tmx_head_sample(void* stream, const void* x, const void* head_w, int M, int D, int V,
+                               int mode, float temperature, uint32_t seed_hi, uint32_t seed_lo,
+                               const int32_t* step, const int32_t* forbidden, int n_forbidden,
+                               const int32_t* eos, int n_eos, int32_t* token_buffer, float* logprobs,
+                               uint8_t* done, int buf_len, float* logits_out, void* workspace) {
+  if (!x || !head_w || !step || !token_buffer || !done || !workspace) return TMX_ERR_ARG;
+  if ((n_forbidden > 0 && !forbidden) || (n_eos > 0 && !eos)) return TMX_ERR_ARG;
+  if (mode != TMX_SAMPLE_GREEDY && mode != TMX_SAMPLE_TOP_P) return TMX_ERR_UNSUPPORTED;
+  HeadArgs a = {};
+  a.x = (const uint16_t*)x;
+  a.w = (const uint16_t*)head_w;
+  a.M = M; a.D = D; a.V = V;
+  a.mode = mode;
+  a.temperature = temperature;
+  a.k0 = seed_hi; a.k1 = seed_lo;
+  a.step = step;
+  a.forbidden = forbidden; a.n_forbidden = n_forbidden;
+  a.logits_out = logits_out;
+  const size_t nwg = (V + 127) / 128;
+  a.part_f = (float*)workspace;
+  a.part_i = (int32_t*)((float*)workspace + (size_t)M * nwg * 4);
+  a.token_buffer = token_buffer;
+  a.logprobs = logprobs;
+  a.done = done;
+  a.eos = eos; a.n_eos = n_eos;
+  a.buf_len = buf_len;
+  return head_sample((hipStream_t)stream, a);
+}

@@ -1,0 +1,122 @@
+// Argument blocks and host-side launch functions shared by the translation units.
+#pragma once
+#include "tmx_common.h"
+
+namespace tmx {
+
+struct QLinearArgs {
+  const uint16_t* x;       // [M, K] bf16
+  int ldx;
+  const uint4* qw;         // packed int4 tiles
+  const uint16_t* scales;  // [N/32][K/G][32] bf16
+  const uint16_t* a_t;     // LoRA A transposed [Rpad, K] bf16 (may be null)
+  uint16_t* y;             // [M, N] bf16 base output
+  int ldy;
+  uint16_t* t;             // [M, Rpad] bf16 LoRA projection output
+  int ldt;
+  int M, K, N, G, Rpad;
+  int n_main_blocks;
+};
+
+struct RowNormArgs {
+  // source of the row: either an embedding gather (embed != null) or y (+ LoRA) (+ residual)
+  const uint16_t* embed;        // [V, D]
+  const int32_t* token_buffer;  // [B, L]
+  const int32_t* step;          // device scalar: column of token_buffer to read
+  int buf_len;
+  const uint16_t* y;            // [M, D] base projection output
+  const uint16_t* t;            // [M, ldt] LoRA projection (null: none)
+  int ldt;
+  const uint16_t* lora_b;       // [r, D]
+  int r;
+  float ls;
+  const uint16_t* residual;     // [M, D] (null: none)
+  uint16_t* x_out;              // [M, D] new residual stream (null: not stored)
+  const uint16_t* norm_w;       // [D] (null: no norm output)
+  uint16_t* xn_out;             // [M, D]
+  int D;
+  float eps;
+  int family;
+};
+
+struct RopeArgs {
+  const uint16_t* qkv;   // [B, (N + 2 Kh) * H] base projection output
+  const uint16_t* t;     // [B, ldt]: x.A_q | x.A_k | x.A_v (null: no LoRA)
+  int ldt;
+  const uint16_t* lora_b;  // [r, (N + 2 Kh) * H]
+  int r;
+  float ls;
+  const uint16_t* q_norm_w;  // [H] (Qwen3) or null
+  const uint16_t* k_norm_w;
+  const int32_t* positions;  // [B, L]
+  const int32_t* step;
+  int buf_len;
+  uint16_t* q_out;   // [B, N * H]
+  uint16_t* kcache;  // [B, C, Kh, H]
+  uint16_t* vcache;
+  int N, Kh, H, C;
+  float theta, eps;
+  int family;
+};
+
+struct SwigluArgs {
+  const uint16_t* gu;  // [M, 2F]: gate columns then up columns
+  const uint16_t* t;   // [M, ldt]: x.A_gate | x.A_up
+  int ldt;
+  const uint16_t* lora_b;  // [r, 2F]
+  int r;
+  float ls;
+  uint16_t* act;  // [M, F]
+  int F;
+};
+
+struct AttnArgs {
+  const uint16_t* q;       // [B, N * H] bf16 (already rotated)
+  const uint16_t* kcache;  // [B, C, Kh, H]
+  const uint16_t* vcache;
+  const uint8_t* input_mask;  // [B, L], 1 = real token
+  const int32_t* step;        // device scalar: newest valid cache slot
+  int buf_len;
+  uint16_t* out;     // [B, N * H] bf16
+  float* partial;    // [B, Kh, nsplit, G, H + 2] (nsplit > 1)
+  int B, N, Kh, C, nsplit, chunk;
+  float scale;
+};
+
+struct HeadArgs {
+  const uint16_t* x;  // [M, D] final-normed hidden states
+  const uint16_t* w;  // [V, D]
+  int M, D, V;
+  int mode;
+  float temperature;
+  uint32_t k0, k1;
+  const int32_t* step;
+  const int32_t* forbidden;
+  int n_forbidden;
+  float* logits_out;  // [M, V] raw f32 logits, optional
+  float* part_f;      // [M][nwg][4] = max, sumexp, best key, best z
+  int32_t* part_i;    // [M][nwg]
+  int nwg;
+  // finalize
+  int32_t* token_buffer;
+  float* logprobs;
+  uint8_t* done;
+  const int32_t* eos;
+  int n_eos;
+  int buf_len;
+};
+
+
+int row_norm(hipStream_t st, const RowNormArgs& a, int M);
+int rope_kvwrite(hipStream_t st, const RopeArgs& a, int B);
+int swiglu(hipStream_t st, const SwigluArgs& a, int M);
+int advance_step(hipStream_t st, int32_t* step);
+int gqa_decode(hipStream_t st, AttnArgs a, int H);
+size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
+int head_sample(hipStream_t st, HeadArgs a);
+size_t head_partial_bytes(int M, int V);
+int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
+                 const void* a_t, void* y, int ldy, void* t, int ldt, int M, int K, int N, int G,
+                 int Rpad);
+
+}  // namespace tmx

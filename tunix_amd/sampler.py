@@ -1,0 +1,312 @@
+"""Sampler with the reference's call surface, running the decode loop on the GPU.
+
+Mirrors tunix/generate/sampler.py:205 ``Sampler`` (constructor :208-214,
+``__call__`` :795-1080, ``transformer_state`` :267-359, ``update_params`` :361-392,
+``tokenize`` :511-518, ``dtype`` :394-400) and base_sampler.py:59 ``BaseSampler``.
+The jitted prefill / while_loop pair is replaced by ``tmx_decode_steps``: prompt
+positions are walked through the same single-token step without the head (cache
+fill), then every generation step runs with the fused head + token selection.
+"""
+import ctypes
+import warnings
+
+import numpy as np
+import torch
+
+from tunix_amd import _lib
+from tunix_amd import utils
+from tunix_amd.configs import CacheConfig, SamplerOutput
+from tunix_amd.model import DecodeState, SAMPLE_GREEDY, SAMPLE_TOP_P
+
+_REQUIRED_TOKENIZER_METHODS = ('encode', 'decode', 'bos_id', 'eos_id', 'pad_id')
+
+
+class TokenizerAdapter:
+  """Duck-typed tokenizer wrapper (tunix/generate/tokenizer_adapter.py:34): accepts
+  any object with encode / decode / bos_id / eos_id / pad_id."""
+
+  def __init__(self, tokenizer):
+    missing = [m for m in _REQUIRED_TOKENIZER_METHODS if not hasattr(tokenizer, m)]
+    if missing:
+      raise ValueError(
+          'Your tokenizer should have the following methods: '
+          '`["encode", "decode", "bos_id", "eos_id", "pad_id"]`. Received: '
+          f'`type(tokenizer)` = {type(tokenizer)}, with missing methods: {missing}.')
+    self._tokenizer = tokenizer
+
+  def encode(self, text, **kw):
+    return self._tokenizer.encode(text, **kw)
+
+  def decode(self, ids, **kw):
+    return self._tokenizer.decode(ids, **kw)
+
+  def bos_id(self):
+    return self._tokenizer.bos_id()
+
+  def eos_id(self):
+    return self._tokenizer.eos_id()
+
+  def pad_id(self):
+    return self._tokenizer.pad_id()
+
+  def dedup_bos_ids(self, ids):
+    i = 0
+    while i < len(ids) - 1 and ids[i] == ids[i + 1] == self.bos_id():
+      i += 1
+    return ids[i:]
+
+
+def _seed_key(seed):
+  """jax.random.PRNGKey(int) as (hi32, lo32); a 2-word key passes through."""
+  if seed is None:
+    seed = 0
+  if isinstance(seed, (int, np.integer)):
+    seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+    return seed >> 32, seed & 0xFFFFFFFF
+  arr = np.asarray(seed).astype(np.uint32).reshape(-1)
+  if arr.size != 2:
+    raise ValueError('seed must be an int or a 2-word key')
+  return int(arr[0]), int(arr[1])
+
+
+class Sampler:
+  """Sampler for an int4 QLoRA decoder resident on one MI355X."""
+
+  # decode steps enqueued between two host checks of the `done` flags
+  CHECK_EVERY = 32
+
+  def __init__(self, transformer, tokenizer, cache_config: CacheConfig, image_processor=None):
+    if image_processor is not None:
+      raise NotImplementedError('image inputs are outside this decode path')
+    self.tokenizer = tokenizer if isinstance(tokenizer, TokenizerAdapter) else TokenizerAdapter(tokenizer)
+    self.cache_config = cache_config
+    self._transformer = transformer
+    c = transformer.config
+    if (cache_config.num_layers, cache_config.num_kv_heads, cache_config.head_dim) != (
+        c.num_layers, c.num_kv_heads, c.head_dim):
+      raise ValueError('cache_config does not match the transformer configuration')
+    self._lib = _lib.lib()  # raises if the HIP library is missing
+    self._cache = None
+    self._workspace = None
+    self.eos_ids = None
+    self.last_step_logits = None
+
+  # -- reference surface -----------------------------------------------------
+  @property
+  def transformer(self):
+    return self._transformer
+
+  @property
+  def transformer_state(self):
+    """Flat dict of parameters: LoRA tensors by the reference's parameter paths."""
+    return self._transformer.lora_state()
+
+  @transformer_state.setter
+  def transformer_state(self, state):
+    self._transformer.update_lora(state)
+
+  def update_params(self, updated_weights, filter_types=None):
+    """LoRA weight sync between rollouts (tunix/rl/rl_cluster.py:1279-1294 passes the
+    LoRA-filtered state).  New tensors are cast to the rollout precision (bf16)."""
+    del filter_types
+    flat = {k: torch.as_tensor(v) for k, v in dict(updated_weights).items()}
+    merged = dict(self._transformer.lora_state())
+    unknown = set(flat) - set(merged)
+    if unknown:
+      raise ValueError(f'New state must have the same structure as the old state. Unknown: {sorted(unknown)[:3]}')
+    merged.update(flat)
+    self._transformer.update_lora(merged)
+
+  @property
+  def dtype(self):
+    return self._transformer.dtype
+
+  def tokenize(self, input_string):
+    ids = self.tokenizer.encode(input_string)
+    bos = [self.tokenizer.bos_id()] if self.tokenizer.bos_id() else []
+    return np.array(self.tokenizer.dedup_bos_ids(bos + list(ids)), dtype=np.int32)
+
+  def delete_cache(self):
+    self._cache = None
+    self._workspace = None
+
+  def reinitialize_cache(self):
+    pass
+
+  # -- state ----------------------------------------------------------------
+  def init_sample_state(self, all_input_ids, total_sampling_steps, include_logits,
+                        forbidden_token_ids, temperature, top_p, top_k, seed, beam_size=None,
+                        include_logprobs=False, prompt_lengths=None):
+    """Device-side _SamplingState (tunix/generate/sampler.py:402-509)."""
+    if beam_size is not None:
+      raise NotImplementedError('beam search is outside this decode path')
+    dev = self._transformer.device
+    ids = np.asarray(all_input_ids, dtype=np.int32)
+    b, p = ids.shape
+    pad = self.tokenizer.pad_id()
+    token_buffer = np.full((b, total_sampling_steps), pad, dtype=np.int32)
+    token_buffer[:, :p] = ids
+    input_mask = np.ones((b, total_sampling_steps), dtype=bool)
+    if prompt_lengths is not None:
+      lens = np.asarray(prompt_lengths).reshape(-1, 1)
+      input_mask[:, :p] = np.arange(p)[None, :] >= (p - lens)
+    else:
+      input_mask[:, :p] = ids != pad
+    positions = utils.build_positions_from_mask(input_mask)
+    c = self._transformer.config
+    need = (c.num_layers, 2, b, self.cache_config.cache_size, c.num_kv_heads, c.head_dim)
+    if self._cache is None or tuple(self._cache.shape) != need:
+      self._cache = None
+      self._cache = self._transformer.init_cache(b, self.cache_config.cache_size)
+    else:
+      self._cache.zero_()
+    st = {
+        'token_buffer': torch.from_numpy(token_buffer).to(dev),
+        'input_mask_host': input_mask,
+        'input_mask': torch.from_numpy(input_mask.astype(np.uint8)).to(dev),
+        'positions_host': positions,
+        'positions': torch.from_numpy(positions.astype(np.int32)).to(dev),
+        'done': torch.zeros(b, dtype=torch.uint8, device=dev),
+        'logprobs': torch.zeros(b, total_sampling_steps, dtype=torch.float32, device=dev)
+                    if include_logprobs else None,
+        'step': torch.zeros(1, dtype=torch.int32, device=dev),
+        'cache': self._cache,
+        'num_input_tokens': p,
+        'total_sampling_steps': total_sampling_steps,
+        'sampling_mode': 'greedy' if top_p is None else 'top_p',
+        'temperature': float(temperature),
+        'top_p': top_p, 'top_k': top_k,
+        'seed': _seed_key(seed),
+        'forbidden': torch.tensor(list(forbidden_token_ids), dtype=torch.int32, device=dev)
+                     if forbidden_token_ids else None,
+        'eos': torch.tensor(np.asarray(self.eos_ids).reshape(-1), dtype=torch.int32, device=dev),
+        'logits': torch.zeros(b, c.vocab_size, dtype=torch.float32, device=dev) if include_logits else None,
+    }
+    return st
+
+  def _c_state(self, st):
+    b, total = st['token_buffer'].shape
+    ws_bytes = self._lib.tmx_decode_workspace_bytes(
+        ctypes.byref(self._transformer.desc()), b, self.cache_config.cache_size)
+    if self._workspace is None or self._workspace.numel() < ws_bytes:
+      self._workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=self._transformer.device)
+    s = DecodeState()
+    s.batch, s.buf_len, s.cache_size = b, total, self.cache_config.cache_size
+    s.token_buffer, s.positions = st['token_buffer'].data_ptr(), st['positions'].data_ptr()
+    s.input_mask, s.done, s.step = st['input_mask'].data_ptr(), st['done'].data_ptr(), st['step'].data_ptr()
+    s.logprobs = st['logprobs'].data_ptr() if st['logprobs'] is not None else None
+    s.kv_cache = st['cache'].data_ptr()
+    s.sampling_mode = SAMPLE_GREEDY if st['sampling_mode'] == 'greedy' else SAMPLE_TOP_P
+    s.temperature = st['temperature']
+    s.top_p = 1.0 if st['top_p'] is None else float(st['top_p'])
+    s.top_k = int(st['top_k']) if st['top_k'] else 0
+    s.seed_hi, s.seed_lo = st['seed']
+    s.eos_ids, s.n_eos = st['eos'].data_ptr(), st['eos'].numel()
+    if st['forbidden'] is not None:
+      s.forbidden, s.n_forbidden = st['forbidden'].data_ptr(), st['forbidden'].numel()
+    s.logits_out = st['logits'].data_ptr() if st['logits'] is not None else None
+    s.workspace, s.workspace_bytes = self._workspace.data_ptr(), self._workspace.numel()
+    return s
+
+  def run_steps(self, st, n_steps, sample=True):
+    """Enqueues n decode-loop iterations on the current stream (no host sync)."""
+    if n_steps <= 0:
+      return
+    cs = self._c_state(st)
+    rc = self._lib.tmx_decode_steps(ctypes.byref(self._transformer.desc()), ctypes.byref(cs),
+                                    _lib.stream(), int(n_steps), 1 if sample else 0)
+    _lib.check(rc, 'tmx_decode_steps')
+
+  # -- the call ---------------------------------------------------------------
+  def __call__(self, input_strings=None, max_generation_steps=0, max_prompt_length=None, echo=False,
+               return_logits=False, return_logprobs=False, eos_tokens=None, forbidden_tokens=None,
+               temperature=0.0, top_p=None, top_k=None, beam_size=None, seed=None, pad_output=False,
+               images=None, audios=None, max_audio_length=None, max_audio_clips=None, *,
+               prompt_token_ids=None):
+    if images is not None or audios is not None:
+      raise NotImplementedError('image / audio inputs are outside this decode path')
+    self.eos_ids = np.array(list(eos_tokens) if eos_tokens else [self.tokenizer.eos_id()])
+    exact_input = prompt_token_ids is not None
+    tokens = utils.resolve_prompt_tokens(
+        input_strings, prompt_token_ids, self.tokenize,
+        max_generation_steps=max_generation_steps,
+        max_total_length=self.cache_config.cache_size,
+        max_length_name='cache_size',
+        single_output_per_row=beam_size is None)
+    if beam_size is not None:
+      raise NotImplementedError('beam search is outside this decode path')
+    forbidden = tuple(forbidden_tokens) if forbidden_tokens else None
+    all_input_ids, prompt_lengths, max_prompt_length = utils.left_pad_prompt_tokens(
+        tokens, max_prompt_length, self.tokenizer.pad_id(),
+        max_allowed_length=self.cache_config.cache_size - max_generation_steps)
+    total = max_prompt_length + max_generation_steps
+    if total > self.cache_config.cache_size:
+      raise ValueError(f'Total sampling steps {total} must be less than the cache size'
+                       f' {self.cache_config.cache_size}.')
+    st = self.init_sample_state(
+        all_input_ids, total, return_logits, forbidden, temperature, top_p, top_k, seed, beam_size,
+        include_logprobs=return_logprobs, prompt_lengths=prompt_lengths if exact_input else None)
+    p = max_prompt_length
+    logits_steps = []
+    if max_generation_steps > 0:
+      # cache fill over prompt columns 0 .. P-2, then P-1 produces generated token #1
+      self.run_steps(st, p - 1, sample=False)
+      remaining = max_generation_steps
+      while remaining > 0:
+        n = 1 if return_logits else min(self.CHECK_EVERY, remaining)
+        self.run_steps(st, n, sample=True)
+        remaining -= n
+        if return_logits:
+          logits_steps.append(st['logits'].clone())
+        if remaining > 0 and bool(st['done'].all().item()):
+          break
+    token_buffers = st['token_buffer'].cpu().numpy()
+    logprob_buffers = st['logprobs'].cpu().numpy() if return_logprobs else None
+    if return_logits and logits_steps:
+      self.last_step_logits = logits_steps[-1]
+      gen_logits = torch.stack(logits_steps, dim=1).cpu().numpy()  # [B, steps, V]
+    else:
+      gen_logits = None
+    pad = self.tokenizer.pad_id()
+
+    def bounds(row, prompt_length):
+      if not echo:
+        start = p
+      elif exact_input:
+        start = p - int(prompt_length)
+      else:
+        start = utils.find_first_non_pad_idx(row, pad)
+      end = utils.find_first_eos_idx(row[p:], self.eos_ids) + p
+      return start, end
+
+    out_tokens, out_logits, out_logprobs = [], [], []
+    max_len = total if echo else max_generation_steps
+    for i, row in enumerate(token_buffers):
+      start, end = bounds(row, prompt_lengths[i])
+      toks = row[start:end]
+      if pad_output:
+        toks = utils.pad_to_length(toks, max_len, pad)
+      out_tokens.append(toks)
+      if gen_logits is not None:
+        lg = gen_logits[i][: max(end - p, 0)]
+        out_logits.append(lg)
+      if return_logprobs:
+        lp = logprob_buffers[i][start:end]
+        if pad_output:
+          lp = np.pad(lp, (0, max_len - len(lp)), mode='constant', constant_values=0.0)
+        out_logprobs.append(lp.tolist())
+    if pad_output:
+      lengths = [bounds(r, prompt_lengths[i])[1] - bounds(r, prompt_lengths[i])[0]
+                 for i, r in enumerate(token_buffers)]
+      decoded = [self.tokenizer.decode(t[:n].tolist()) for t, n in zip(out_tokens, lengths)]
+      out_tokens = np.stack(out_tokens) if out_tokens else out_tokens
+    else:
+      decoded = [self.tokenizer.decode(t.tolist()) for t in out_tokens]
+    return SamplerOutput(
+        text=decoded,
+        logits=out_logits if return_logits else [],
+        tokens=out_tokens,
+        padded_prompt_tokens=all_input_ids,
+        logprobs=out_logprobs if return_logprobs else None,
+        prompt_lengths=prompt_lengths,
+    )
