@@ -1,0 +1,249 @@
+"""Benchmark of the decode path: generated tokens/s of an int4 QLoRA rollout on one MI355X.
+
+A "step" is one decode-loop iteration over the whole batch (one new token per
+sequence).  Default workload: Llama-3.1-8B shape, 64 sequences (8 prompts x 8
+samples), 256-token prompts, temperature 0.9, top-p 1.0, per-token logprobs,
+bf16 KV cache.  The timed region covers the generation steps that follow the
+warmup steps of the same rollout, so the context grows from 256 + warmup towards 767
+(mean about 512).  Prints one JSON line.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # name: (config factory, batch, prompt, new tokens, group, rank, temperature, top_p)
+    'llama3.1-8b-grpo': ('llama3p1_8b', 64, 256, 512, 64, 16, 0.9, 1.0),
+    'llama3.2-1b-b1': ('llama3p2_1b', 1, 256, 512, 64, 16, 1.0, 1.0),
+    'toy': ('toy', 4, 32, 32, 64, 8, 0.9, 1.0),
+}
+
+CLASS_NAMES = ['row_norm', 'qkv_linear', 'rope_kvwrite', 'attention', 'o_linear', 'gate_up_linear',
+               'swiglu', 'down_linear', 'head_sample', 'advance_step']
+
+
+def linear_bytes(pl, batch):
+  """int4 + scales + LoRA A, B (+ activations in and out, counted for the GEMM regime)."""
+  b = pl.k * pl.n // 2 + (pl.k // pl.group) * pl.n * 2
+  if pl.lora_a_t is not None:
+    b += 2 * pl.rank * (pl.k * len(pl.seg_cols) + pl.n)
+  return b + batch * (pl.k + pl.n) * 2
+
+
+def cpu_baseline(workload, n_layers=2):
+  """One decode step of the CPU oracle (dequantise -> bf16 matmul, attention over the whole
+  cache, f32 log-softmax) at the workload's shapes on `n_layers` layers + head, scaled to
+  the full depth.  Reported beside the GPU number, not a target."""
+  import torch
+  from oracle import model as OM
+  from oracle import masks as OMK
+  from oracle import sampling as OS
+  name, batch, prompt, new, group, rank, temp, _ = WORKLOADS[workload]
+  from tunix_amd.model import ModelConfig
+  c = getattr(ModelConfig, name)()
+  full_layers = c.num_layers
+  # the layers are timed with a tiny vocabulary (the embedding is only gathered); the head
+  # matrix of the real shape is a tiled random block (values do not affect the timing)
+  ocfg = OM.Config(c.family, min(n_layers, full_layers), 32, c.embed_dim, c.hidden_dim,
+                   c.num_heads, c.head_dim, c.num_kv_heads, c.rope_theta, c.norm_eps, True)
+  w = OM.random_weights(ocfg, 0, group, rank, 2.0 * rank,
+                        ('q', 'k', 'v', 'o', 'gate', 'up', 'down'))
+  dec = OM.Decoder(ocfg, w)
+  cache_size = prompt + new
+  step = prompt + new // 2
+  cache = OM.init_cache(ocfg, batch, cache_size)
+  rng = np.random.default_rng(0)
+  for lc in cache.values():
+    lc['end_index'][:] = step
+    lc['k'][:, :step] = rng.standard_normal((batch, step, c.num_kv_heads, c.head_dim), dtype=np.float32)
+    lc['v'][:, :step] = lc['k'][:, :step]
+  block = (rng.standard_normal((c.embed_dim, 1002), dtype=np.float32) * np.float32(0.02))
+  reps = -(-c.vocab_size // 1002)
+  head = np.ascontiguousarray(np.tile(block, (1, reps))[:, :c.vocab_size])
+  x = rng.standard_normal((batch, 1, c.embed_dim), dtype=np.float32)
+  pos = np.full((batch, 1), step, np.int32)
+  mask = OMK.compute_attention_masks(step, cache_size, np.zeros((batch, cache_size), bool))
+  from oracle import layers as L
+  t_layers0 = time.perf_counter()
+  for i, lw in enumerate(dec.w['layers']):
+    lc, a = dec._attn(lw, dec._norm(x, lw['norm1']), pos, cache[f'layer_{i}'], mask)
+    h = dec.pol.r(a + x)
+    m = L.swiglu_mlp(dec._norm(h, lw['norm2']), lw['gate'], lw['up'], lw['down'], dec.pol, 'reference')
+    x = dec.pol.r(h + m)
+  t_layers = time.perf_counter() - t_layers0
+  t_head0 = time.perf_counter()
+  xn = dec._norm(x, dec.w['final_norm'])
+  logits = dec.pol.r(xn @ head)
+  OS.log_softmax(logits[:, -1] / np.float32(temp))
+  t_head = time.perf_counter() - t_head0
+  step_s = t_layers * full_layers / ocfg.num_layers + t_head
+  return {
+      'value': batch / step_s,
+      'unit': 'tokens/s',
+      'cores': int(os.environ.get('OMP_NUM_THREADS', torch.get_num_threads())),
+      'kind': 'port',
+      'sample': (f'CPU restatement (numpy), not tunix/JAX: 1 decode step at context {step}, '
+                 f'{ocfg.num_layers} of {full_layers} layers timed ({t_layers:.2f} s) and scaled, '
+                 f'+ head ({t_head:.2f} s); os.cpu_count()={os.cpu_count()}'),
+  }
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument('--gpus', type=int, default=1)
+  ap.add_argument('--steps', type=int, default=496)
+  ap.add_argument('--warmup', type=int, default=16)
+  ap.add_argument('--workload', default='llama3.1-8b-grpo', choices=sorted(WORKLOADS))
+  ap.add_argument('--no-cpu-baseline', action='store_true')
+  ap.add_argument('--no-profile', action='store_true')
+  args = ap.parse_args()
+  if args.gpus != 1:
+    print('bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1',
+          file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+  from tunix_amd import _lib
+  from tunix_amd.configs import CacheConfig
+  from tunix_amd.model import ModelConfig, QLoRAModel
+  from tunix_amd.sampler import Sampler
+  sys.path.insert(0, os.path.join(ROOT, 'tests'))
+
+  name, batch, prompt, new, group, rank, temp, top_p = WORKLOADS[args.workload]
+  if args.steps + args.warmup > new:
+    print(f'bench.py: steps + warmup must be <= {new} new tokens of the workload', file=sys.stderr)
+    sys.exit(2)
+  cfg = getattr(ModelConfig, name)()
+  torch.cuda.set_device(0)
+  model = QLoRAModel.random_init(cfg, seed=0, group=group, lora_rank=rank, lora_alpha=2.0 * rank)
+  cache_size = prompt + new
+
+  class _Tok:  # ids only: the benchmark feeds token ids and never decodes text
+    def encode(self, s): return [int(t) for t in s.split()]
+    def decode(self, ids): return ''
+    def pad_id(self): return 0
+    def bos_id(self): return 1
+    def eos_id(self): return -1
+
+  sampler = Sampler(model, _Tok(), CacheConfig(cache_size, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
+  sampler.eos_ids = np.array([-1])  # unreachable: every row runs the full length
+  rng = np.random.default_rng(0)
+  n_prompts = max(batch // 8, 1)
+  base = rng.integers(3, cfg.vocab_size, (n_prompts, prompt)).astype(np.int32)
+  ids = np.repeat(base, batch // n_prompts, axis=0)  # G samples of a prompt are consecutive rows
+
+  def fresh_state():
+    st = sampler.init_sample_state(ids, prompt + new, False, None, temp, top_p, None, 0,
+                                   include_logprobs=True, prompt_lengths=np.full(batch, prompt))
+    sampler.run_steps(st, prompt - 1, sample=False)  # cache fill over the prompt (untimed)
+    return st
+
+  st = fresh_state()
+  sampler.run_steps(st, args.warmup, sample=True)
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  sampler.run_steps(st, args.steps, sample=True)
+  torch.cuda.synchronize()
+  dt = time.perf_counter() - t0
+  toks = st['token_buffer'][:, prompt:prompt + args.warmup + args.steps]
+  assert int(st['step'].item()) == prompt - 1 + args.warmup + args.steps
+  assert bool(((toks >= 0) & (toks < cfg.vocab_size)).all().item())
+  lps = st['logprobs'][:, prompt:prompt + args.warmup + args.steps]
+  assert bool(torch.isfinite(lps).all().item()) and bool((lps <= 0).all().item())
+
+  result = {
+      'metric': 'generated tokens/s at 1 GPU, int4 QLoRA 8B rollout (decode)',
+      'value': batch * args.steps / dt,
+      'unit': 'tokens/s',
+      'n_gpus': 1,
+      'steps': args.steps,
+      'warmup': args.warmup,
+      'ms_per_step': dt / args.steps * 1e3,
+      'higher_is_better': True,
+      'scaling': 'weak',
+      'vs_baseline': None,
+      'dtype': 'bf16 activations / int4 weights / f32 accumulate',
+      'data': 'synthetic (random-init weights, uniform-random prompt ids)',
+      'config': {
+          'workload': args.workload,
+          'shape': name, 'sequences': batch, 'prompt_len': prompt, 'new_tokens': new,
+          'quant': f'int4 group {group}', 'lora_rank': rank, 'temperature': temp, 'top_p': top_p,
+          'context_range': [prompt - 1 + args.warmup, prompt - 1 + args.warmup + args.steps],
+      },
+  }
+
+  # Whole-step algorithmic bytes at the mean context of the timed region.
+  wbytes, hbytes = model.weight_bytes()
+  s_mean = prompt + args.warmup + args.steps / 2.0
+  kv_per_tok = cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * 2 * 2
+  step_bytes = wbytes + hbytes + batch * s_mean * kv_per_tok
+  result['step_hbm'] = {'algorithmic_bytes': step_bytes,
+                        'achieved_GBps': step_bytes / (dt / args.steps) / 1e9,
+                        'frac_of_8TBps': step_bytes / (dt / args.steps) / 8e12}
+
+  if not args.no_profile:
+    # Replay the same rollout with HIP events around every launch, sampling every 8th step.
+    lib = _lib.lib()
+    st = fresh_state()
+    sampler.run_steps(st, args.warmup, sample=True)
+    ms = np.zeros(len(CLASS_NAMES), np.float32)
+    cnt = np.zeros(len(CLASS_NAMES), np.int32)
+    tot_ms = np.zeros_like(ms)
+    tot_cnt = np.zeros_like(cnt)
+    ctx_sum, ctx_n = 0.0, 0
+    done_steps = 0
+    while done_steps < args.steps:
+      skip = min(7, args.steps - done_steps)
+      sampler.run_steps(st, skip, sample=True)
+      done_steps += skip
+      if done_steps >= args.steps:
+        break
+      ctx_sum += prompt + args.warmup + done_steps
+      ctx_n += 1
+      cs = sampler._c_state(st)
+      rc = lib.tmx_decode_steps_profiled(ctypes.byref(model.desc()), ctypes.byref(cs), _lib.stream(), 1, 1,
+                                         ms.ctypes.data_as(ctypes.c_void_p), cnt.ctypes.data_as(ctypes.c_void_p))
+      _lib.check(rc, 'tmx_decode_steps_profiled')
+      tot_ms += ms
+      tot_cnt += cnt
+      done_steps += 1
+    per_step = tot_ms / max(ctx_n, 1)
+    result['kernel_ms_per_step'] = {n: round(float(v), 4) for n, v in zip(CLASS_NAMES, per_step)}
+    dom = int(np.argmax(tot_ms))
+    avg_ms = float(tot_ms[dom] / max(tot_cnt[dom], 1))
+    layer0 = model.layers[0]
+    ctx = ctx_sum / max(ctx_n, 1)
+    alg = {
+        'qkv_linear': linear_bytes(layer0['qkv'], batch), 'o_linear': linear_bytes(layer0['o'], batch),
+        'gate_up_linear': linear_bytes(layer0['gate_up'], batch),
+        'down_linear': linear_bytes(layer0['down'], batch),
+        'attention': batch * ctx * cfg.num_kv_heads * cfg.head_dim * 2 * 2,
+        'head_sample': hbytes,
+    }
+    if CLASS_NAMES[dom] in alg:
+      a = alg[CLASS_NAMES[dom]] / (avg_ms * 1e-3) / 1e9
+      result['roofline'] = {'bound': 'hbm', 'achieved': a, 'peak': 8000.0, 'unit': 'GB/s',
+                            'frac': a / 8000.0, 'traffic': None, 'kernel': CLASS_NAMES[dom],
+                            'avg_launch_ms': avg_ms, 'algorithmic_bytes_per_launch': alg[CLASS_NAMES[dom]]}
+    result['roofline_all'] = {
+        n: {'avg_launch_ms': float(tot_ms[i] / max(tot_cnt[i], 1)),
+            'achieved_GBps': alg[n] / (float(tot_ms[i] / max(tot_cnt[i], 1)) * 1e-3) / 1e9,
+            'frac': alg[n] / (float(tot_ms[i] / max(tot_cnt[i], 1)) * 1e-3) / 8e12}
+        for i, n in enumerate(CLASS_NAMES) if n in alg and tot_cnt[i] > 0}
+
+  if not args.no_cpu_baseline:
+    del st
+    result['cpu_baseline'] = cpu_baseline(args.workload)
+  print(json.dumps(result))
+
+
+if __name__ == '__main__':
+  main()

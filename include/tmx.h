@@ -42,6 +42,9 @@ extern "C" {
 #define TMX_FAMILY_LLAMA3 0
 #define TMX_FAMILY_QWEN3 1
 
+#define TMX_MAX_RPAD 128   /* widest padded LoRA projection (sum of fused ranks, rounded up to 32) */
+#define TMX_MAX_SPLITS 16  /* most K-slices a projection is split into */
+
 #define TMX_SAMPLE_GREEDY 0
 #define TMX_SAMPLE_TOP_P 1
 
@@ -54,15 +57,26 @@ int tmx_abi_version(void);
 int tmx_int4_dequant(void* stream, const void* qweight, const void* scales, void* w_out, int K, int N,
                      int G);
 
-/* y[M, N] = bf16(x[M, K] . dequant(qweight)) (+ LoRA delta) (+ residual).
+/* y[M, N] = bf16(x[M, K] . dequant(qweight)) (+ LoRA delta) (+ residual), M <= 128.
  * Replaces the qwix-wrapped Einsum / nnx.Linear call: tunix/models/llama3/model.py:216-218,
  * :489-496; tunix/models/qwen3/model.py:389-393, :1199-1208.
  *   lora_a_t : A transposed and zero-padded, bf16 [r_pad, K], r_pad % 32 == 0 (NULL: no LoRA)
- *   lora_b   : bf16 [r, N];  t_ws: bf16 [M, r_pad] workspace receiving x . A
- *   residual : bf16 [M, N] or NULL; added after the LoRA delta, in bf16 */
+ *   lora_b   : bf16 [r, N]
+ *   residual : bf16 [M, N] or NULL; added after the LoRA delta, in bf16
+ *   workspace: tmx_qlora_linear_workspace_bytes(M, K, N) bytes (f32 K-slice planes) */
+size_t tmx_qlora_linear_workspace_bytes(int M, int K, int N);
 int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const void* scales,
-                     const void* lora_a_t, const void* lora_b, const void* residual, void* y, void* t_ws,
-                     int M, int K, int N, int G, int r, int r_pad, float lora_scale);
+                     const void* lora_a_t, const void* lora_b, const void* residual, void* y,
+                     void* workspace, int M, int K, int N, int G, int r, int r_pad, float lora_scale);
+
+/* The matrix product alone, for callers that fuse their own consumer: writes `nsplit` f32
+ * K-slice planes y_part[nsplit][M][N] (their sum is x . dequant(W)) and, with LoRA,
+ * t_part[nsplit][M][TMX_MAX_RPAD] (their sum is x . A).  nsplit in [1, TMX_MAX_SPLITS];
+ * tmx_qlora_linear_num_splits() returns the count the library itself would pick. */
+int tmx_qlora_linear_num_splits(int M, int K, int N);
+int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight, const void* scales,
+                            const void* lora_a_t, float* y_part, float* t_part, int M, int K, int N,
+                            int G, int r_pad, int nsplit);
 
 /* ---- row-wise kernels between the matrix products ------------------------- */
 
@@ -71,28 +85,35 @@ int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const voi
  * in f32 (tunix/models/qwen3/model.py:478-484). */
 int tmx_rmsnorm(void* stream, const void* x, const void* w, void* y, int M, int D, float eps, int family);
 
-/* h = bf16(bf16(y + lora_delta) + residual) -> x_out;  xn_out = RMSNorm(h) * norm_w.
- * lora_delta[m, n] = bf16(bf16(sum_r t[m, r] lora_b[r, n]) * lora_scale); t, residual,
- * x_out, norm_w may be NULL.  Residual wiring of tunix/models/llama3/model.py:546-564,
- * tunix/models/qwen3/model.py:1268-1289. */
-int tmx_lora_residual_rmsnorm(void* stream, const void* y, const void* t, int ldt, const void* lora_b,
-                              int r, float lora_scale, const void* residual, void* x_out,
-                              const void* norm_w, void* xn_out, int M, int D, float eps, int family);
+/* The three consumers below take the output of a projection either as a bf16 tensor
+ * (*_bf16) or as `nsplit` f32 K-slice planes [nsplit][M][N] (*_part) that they sum and round
+ * to bf16 first, and apply the LoRA-B half:
+ *   delta[m, n] = bf16(bf16(sum_r t[m, r] lora_b[r, n]) * lora_scale),
+ *   t[m, r] = bf16(sum_s t_part[s][m][r]), t_part f32 [nsplit][M][ldt] (NULL: no LoRA). */
 
-/* qkv[B, (N + 2 Kh) H] (+ LoRA deltas, t = x.A_q | x.A_k | x.A_v) -> optional per-head
+/* h = bf16(bf16(y + delta) + residual) -> x_out;  xn_out = RMSNorm(h) * norm_w.
+ * residual, x_out, norm_w may be NULL.  Residual wiring of
+ * tunix/models/llama3/model.py:546-564, tunix/models/qwen3/model.py:1268-1289. */
+int tmx_lora_residual_rmsnorm(void* stream, const void* y_bf16, const float* y_part, int nsplit,
+                              const float* t_part, int ldt, const void* lora_b, int r, float lora_scale,
+                              const void* residual, void* x_out, const void* norm_w, void* xn_out, int M,
+                              int D, float eps, int family);
+
+/* qkv[B, (N + 2 Kh) H] (+ deltas, t columns x.A_q | x.A_k | x.A_v) -> optional per-head
  * RMSNorm (Qwen3 q_norm / k_norm), RoPE at positions[b, *step], q_out[B, N H] and the
  * K / V rows of cache slot *step % C.  tunix/models/llama3/model.py:249-270, :348-377;
  * tunix/models/qwen3/model.py:432-453, :559-597. */
-int tmx_rope_kv_write(void* stream, const void* qkv, const void* t, int ldt, const void* lora_b, int r,
-                      float lora_scale, const void* q_norm_w, const void* k_norm_w,
-                      const int32_t* positions, const int32_t* step, int buf_len, void* q_out,
-                      void* kcache, void* vcache, int B, int N, int Kh, int H, int C, float theta,
-                      float eps, int family);
+int tmx_rope_kv_write(void* stream, const void* qkv_bf16, const float* qkv_part, int nsplit,
+                      const float* t_part, int ldt, const void* lora_b, int r, float lora_scale,
+                      const void* q_norm_w, const void* k_norm_w, const int32_t* positions,
+                      const int32_t* step, int buf_len, void* q_out, void* kcache, void* vcache, int B,
+                      int N, int Kh, int H, int C, float theta, float eps, int family);
 
 /* act[M, F] = bf16(silu(gate) * up), gate_up[M, 2F] = gate columns then up columns
- * (+ LoRA deltas, t = x.A_gate | x.A_up).  tunix/models/llama3/model.py:489-496. */
-int tmx_swiglu(void* stream, const void* gate_up, const void* t, int ldt, const void* lora_b, int r,
-               float lora_scale, void* act, int M, int F);
+ * (+ deltas, t columns x.A_gate | x.A_up).  tunix/models/llama3/model.py:489-496. */
+int tmx_swiglu(void* stream, const void* gate_up_bf16, const float* gate_up_part, int nsplit,
+               const float* t_part, int ldt, const void* lora_b, int r, float lora_scale, void* act,
+               int M, int F);
 
 /* ---- GQA decode attention -------------------------------------------------- */
 
@@ -123,7 +144,6 @@ int tmx_head_sample(void* stream, const void* x, const void* head_w, int M, int 
 
 /* ---- whole decode steps ------------------------------------------------------ */
 
-#define TMX_MAX_RPAD 128 /* widest padded LoRA projection (sum of fused ranks, rounded up to 32) */
 
 typedef struct {
   const void* qweight;  /* q4t tiles of the (column-fused) weight [K, N] */
@@ -190,6 +210,24 @@ size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int ca
  * `model`, `state` and model->layers are HOST structures read during the call only. */
 int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
                      int n_steps, int sample);
+
+/* Measurement aid (no counterpart in the reference): the same as tmx_decode_steps, but every
+ * kernel launch is bracketed by HIP events on `stream`; after enqueuing, the call SYNCHRONISES
+ * the stream and adds up the elapsed milliseconds and the launch count per kernel class into
+ * the two HOST arrays of TMX_NUM_KERNEL_CLASSES entries. */
+#define TMX_K_ROWNORM 0  /* embedding gather / residual + LoRA-B + RMSNorm rows */
+#define TMX_K_QKV 1      /* fused q|k|v int4 projection (+ LoRA-A tiles) */
+#define TMX_K_ROPE 2     /* LoRA-B + RoPE + KV-cache write */
+#define TMX_K_ATTN 3     /* GQA decode attention (+ split combine) */
+#define TMX_K_O 4        /* o projection */
+#define TMX_K_GATE_UP 5  /* fused gate|up projection */
+#define TMX_K_SWIGLU 6
+#define TMX_K_DOWN 7     /* down projection */
+#define TMX_K_HEAD 8     /* head + log-softmax + token selection (+ finalize) */
+#define TMX_K_ADVANCE 9
+#define TMX_NUM_KERNEL_CLASSES 10
+int tmx_decode_steps_profiled(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
+                              int n_steps, int sample, float* class_ms_host, int* class_launches_host);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,350 @@
+"""GPU parity of every kernel against the CPU oracle, called through the C ABI."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import int4
+from oracle import layers as L
+from oracle import prng
+from oracle import sampling as OS
+from oracle.bf16 import BF16, bf16_round, bf16_from_bits
+from tunix_amd import _lib
+from tunix_amd import quant
+
+import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+S = _lib.stream
+
+
+def _packed(w, group, loras=None, ls=0.0):
+  return quant.PackedLinear.from_dense([torch.from_numpy(w)], group, G.DEV,
+                                       None if loras is None else [tuple(torch.from_numpy(m) for m in loras)], ls)
+
+
+def test_int4_dequant_bit_exact_exhaustive():
+  T = G.Keep()
+  # every nibble value against 640 distinct bf16 scales, G = 64 and 128
+  scales = bf16_from_bits(np.arange(0x3800, 0x3D00, 2, dtype=np.uint16))  # 640 scales
+  n = scales.size
+  rng = np.random.default_rng(0)
+  for group in (64, 128):
+    k = 2 * group
+    q = rng.integers(-8, 8, (k, n)).astype(np.int8)
+    q[:16, :] = np.arange(-8, 8, dtype=np.int8)[:, None]  # every nibble under every scale
+    s = np.stack([scales, scales[::-1]])
+    qw = quant.pack_q4t(torch.from_numpy(q)).to(G.DEV)
+    st = quant.pack_scales(torch.from_numpy(s).to(torch.bfloat16)).to(G.DEV)
+    out = torch.empty(k, n, dtype=torch.bfloat16, device=G.DEV)
+    G.call('tmx_int4_dequant', S(), G.p(qw), G.p(st), G.p(out), k, n, group)
+    G.sync()
+    np.testing.assert_array_equal(G.host(out), int4.dequantize(q, s, group))
+
+
+@pytest.mark.parametrize('M,K,N,group,r', [
+    (1, 256, 96, 64, 0), (4, 256, 256, 64, 8), (7, 512, 96, 64, 8), (33, 1024, 160, 128, 16),
+    (64, 2048, 1024, 64, 16), (100, 512, 256, 64, 32), (128, 4096, 512, 128, 32), (64, 14336, 256, 64, 16),
+])
+def test_qlora_linear_matches_oracle(M, K, N, group, r):
+  T = G.Keep()
+  rng = np.random.default_rng(M * 7 + N)
+  w = bf16_round(rng.standard_normal((K, N)).astype(np.float32) * 0.02)
+  x = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+  res = bf16_round(rng.standard_normal((M, N)).astype(np.float32))
+  a = b = None
+  if r:
+    a = bf16_round(rng.standard_normal((K, r)).astype(np.float32) * 0.02)
+    b = bf16_round(rng.standard_normal((r, N)).astype(np.float32) * 0.02)
+  pl = _packed(w, group, (a, b) if r else None, 2.0)
+  qo, so = int4.quantize(w, group)
+  lin = L.Linear(q=qo, scale=so, group=group, a=a, b=b, lora_scale=2.0)
+  lib = _lib.lib()
+  ws = torch.empty(lib.tmx_qlora_linear_workspace_bytes(M, K, N), dtype=torch.uint8, device=G.DEV)
+  xt, rs = G.bf(x), G.bf(res)
+  for use_res in (False, True):
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=G.DEV)
+    G.call('tmx_qlora_linear', S(), G.p(xt), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t), G.p(pl.lora_b),
+           G.p(rs) if use_res else None, G.p(y), G.p(ws), M, K, N, group, r, pl.r_pad, 2.0)
+    G.sync()
+    out = lin(x, BF16)
+    ref = bf16_round(out + res) if use_res else out
+    # f32 accumulation order differs: at most one bf16 ulp of the base projection (which the
+    # LoRA / residual adds can turn into several ulps of a small sum), and only rarely
+    base = bf16_round(x @ lin.weight())
+    G.assert_bf16_close(G.host(y), ref, ulps=1.0, extra=G.ulp_bf16(base) if (use_res or r) else 0.0,
+                        min_exact=0.995, what=f'linear {M}x{K}x{N}')
+
+
+def test_qlora_linear_planes_sum_and_rejects():
+  T = G.Keep()
+  rng = np.random.default_rng(1)
+  M, K, N, group = 16, 1024, 128, 64
+  w = bf16_round(rng.standard_normal((K, N)).astype(np.float32) * 0.02)
+  x = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+  pl = _packed(w, group)
+  qo, so = int4.quantize(w, group)
+  lib = _lib.lib()
+  for ns in (1, 2, 4):
+    yp = torch.zeros(ns, M, N, dtype=torch.float32, device=G.DEV)
+    G.call('tmx_qlora_linear_planes', S(), T.bf(x), G.p(pl.qweight), G.p(pl.scales), None, G.p(yp), None,
+           M, K, N, group, 0, ns)
+    G.sync()
+    exact = x.astype(np.float64) @ int4.dequantize(qo, so, group).astype(np.float64)
+    np.testing.assert_allclose(G.host(yp.sum(0)), exact, rtol=0, atol=2e-5 * np.abs(exact).max())
+  assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, 129, K, N, group, 0, 1) == -2  # M > 128
+  assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, M, K, N, 96, 0, 1) == -2      # G not a power of two
+  assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, M, K, N, group, 0, 3) == -2   # empty K-slice
+
+
+@pytest.mark.parametrize('family', [0, 1])
+@pytest.mark.parametrize('M,D', [(1, 256), (5, 2048), (64, 4096), (3, 5120)])
+def test_rmsnorm(family, M, D):
+  T = G.Keep()
+  rng = np.random.default_rng(D + family)
+  x = bf16_round(rng.standard_normal((M, D)).astype(np.float32) * 3)
+  w = bf16_round(rng.uniform(0.5, 1.5, D).astype(np.float32))
+  y = torch.empty(M, D, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_rmsnorm', S(), T.bf(x), T.bf(w), G.p(y), M, D, 1e-5, family)
+  G.sync()
+  ref = (L.rmsnorm_llama3 if family == 0 else L.rmsnorm_qwen3)(x, w, 1e-5, BF16)
+  G.assert_bf16_close(G.host(y), ref, ulps=1.0, min_exact=0.99, what='rmsnorm')
+
+
+@pytest.mark.parametrize('family', [0, 1])
+def test_lora_residual_rmsnorm_planes(family):
+  T = G.Keep()
+  rng = np.random.default_rng(3)
+  M, D, r, ns = 9, 1024, 16, 3
+  yp = rng.standard_normal((ns, M, D)).astype(np.float32)
+  tp = rng.standard_normal((ns, M, 128)).astype(np.float32)
+  b = bf16_round(rng.standard_normal((r, D)).astype(np.float32) * 0.05)
+  res = bf16_round(rng.standard_normal((M, D)).astype(np.float32))
+  w = bf16_round(rng.uniform(0.5, 1.5, D).astype(np.float32))
+  x_out = torch.empty(M, D, dtype=torch.bfloat16, device=G.DEV)
+  xn = torch.empty(M, D, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_lora_residual_rmsnorm', S(), None, T.f32(yp), ns, T.f32(tp), 128, T.bf(b), r, 1.5,
+         T.bf(res), G.p(x_out), T.bf(w), G.p(xn), M, D, 1e-6, family)
+  G.sync()
+  y = bf16_round(yp.sum(0))
+  t = bf16_round(tp.sum(0)[:, :r])
+  d = bf16_round(bf16_round(t @ b) * np.float32(1.5))
+  h = bf16_round(bf16_round(y + d) + res)
+  G.assert_bf16_close(G.host(x_out), h, ulps=1.0, min_exact=0.99, what='residual stream')
+  got_h = G.host(x_out)
+  ref = (L.rmsnorm_llama3 if family == 0 else L.rmsnorm_qwen3)(got_h, w, 1e-6, BF16)
+  G.assert_bf16_close(G.host(xn), ref, ulps=1.0, min_exact=0.99, what='norm of residual')
+
+
+@pytest.mark.parametrize('family,H,N,Kh', [(0, 64, 4, 4), (0, 128, 8, 2), (1, 128, 4, 2), (1, 64, 8, 8)])
+def test_rope_kv_write(family, H, N, Kh):
+  T = G.Keep()
+  rng = np.random.default_rng(H + N)
+  B, C, Lbuf, r, ns, step = 3, 12, 10, 8, 2, 5
+  ntot = (N + 2 * Kh) * H
+  qkv = rng.standard_normal((ns, B, ntot)).astype(np.float32)
+  tp = rng.standard_normal((ns, B, 128)).astype(np.float32)
+  lb = bf16_round(rng.standard_normal((r, ntot)).astype(np.float32) * 0.05)
+  qn = bf16_round(rng.uniform(0.5, 1.5, H).astype(np.float32))
+  kn = bf16_round(rng.uniform(0.5, 1.5, H).astype(np.float32))
+  positions = rng.integers(0, 700, (B, Lbuf)).astype(np.int32)
+  kc = torch.full((B, C, Kh, H), 7.0, dtype=torch.bfloat16, device=G.DEV)
+  vc = torch.full((B, C, Kh, H), 7.0, dtype=torch.bfloat16, device=G.DEV)
+  q_out = torch.empty(B, N * H, dtype=torch.bfloat16, device=G.DEV)
+  theta = 1_000_000.0 if family == 0 else 10_000.0
+  G.call('tmx_rope_kv_write', S(), None, T.f32(qkv), ns, T.f32(tp), 128, T.bf(lb), r, 2.0,
+         T.bf(qn) if family else None, T.bf(kn) if family else None, T.i32(positions),
+         T.i32([step]), Lbuf, G.p(q_out), G.p(kc), G.p(vc), B, N, Kh, H, C, theta, 1e-6, family)
+  G.sync()
+  y = bf16_round(qkv.sum(0))
+  t = bf16_round(tp.sum(0))
+  cols = np.arange(ntot)
+  seg = np.where(cols < N * H, 0, np.where(cols < (N + Kh) * H, 1, 2))
+  d = np.zeros_like(y)
+  for s in range(3):
+    d[:, seg == s] = bf16_round(bf16_round(t[:, s * r:(s + 1) * r] @ lb[:, seg == s]) * np.float32(2.0))
+  y = bf16_round(y + d)
+  q = y[:, :N * H].reshape(B, 1, N, H)
+  k = y[:, N * H:(N + Kh) * H].reshape(B, 1, Kh, H)
+  v = y[:, (N + Kh) * H:].reshape(B, Kh, H)
+  pos = positions[:, step:step + 1]
+  if family:
+    q, k = L.rmsnorm_qwen3(q, qn, 1e-6, BF16), L.rmsnorm_qwen3(k, kn, 1e-6, BF16)
+    q, k = L.rope_qwen3(q, pos, theta, BF16), L.rope_qwen3(k, pos, theta, BF16)
+  else:
+    q, k = L.rope_llama3(q, pos, theta, BF16), L.rope_llama3(k, pos, theta, BF16)
+  # trig of angles up to ~700 rad: GPU and numpy sin/cos agree to ~1e-6 relative of the angle
+  G.assert_bf16_close(G.host(q_out), q.reshape(B, -1), ulps=1.0, extra=2e-3, min_exact=0.97, what='q')
+  kc_h, vc_h = G.host(kc), G.host(vc)
+  G.assert_bf16_close(kc_h[:, step], k[:, 0], ulps=1.0, extra=2e-3, min_exact=0.97, what='k row')
+  np.testing.assert_array_equal(vc_h[:, step], v)
+  others = [i for i in range(C) if i != step]
+  assert np.all(kc_h[:, others] == 7.0) and np.all(vc_h[:, others] == 7.0)
+
+
+@pytest.mark.parametrize('M,F,ns', [(3, 1024, 0), (64, 14336, 2), (5, 768, 1)])
+def test_swiglu(M, F, ns):
+  T = G.Keep()
+  rng = np.random.default_rng(F)
+  r = 16
+  lb = bf16_round(rng.standard_normal((r, 2 * F)).astype(np.float32) * 0.05)
+  act = torch.empty(M, F, dtype=torch.bfloat16, device=G.DEV)
+  if ns == 0:
+    gu = bf16_round(rng.standard_normal((M, 2 * F)).astype(np.float32) * 2)
+    G.call('tmx_swiglu', S(), T.bf(gu), None, 0, None, 0, None, 0, 0.0, G.p(act), M, F)
+    y = gu
+  else:
+    gp = rng.standard_normal((ns, M, 2 * F)).astype(np.float32)
+    tp = rng.standard_normal((ns, M, 128)).astype(np.float32)
+    G.call('tmx_swiglu', S(), None, T.f32(gp), ns, T.f32(tp), 128, T.bf(lb), r, 2.0, G.p(act), M, F)
+    y = bf16_round(gp.sum(0))
+    t = bf16_round(tp.sum(0))
+    dg = bf16_round(bf16_round(t[:, :r] @ lb[:, :F]) * np.float32(2.0))
+    du = bf16_round(bf16_round(t[:, r:2 * r] @ lb[:, F:]) * np.float32(2.0))
+    y = np.concatenate([bf16_round(y[:, :F] + dg), bf16_round(y[:, F:] + du)], axis=1)
+  G.sync()
+  ref = bf16_round(L.silu(y[:, :F], BF16) * y[:, F:])
+  G.assert_bf16_close(G.host(act), ref, ulps=1.0, min_exact=0.98, what='swiglu')
+
+
+@pytest.mark.parametrize('B,N,Kh,H,C,step', [
+    (2, 4, 4, 64, 64, 40), (3, 8, 2, 64, 96, 95), (2, 8, 4, 64, 33, 0), (4, 32, 8, 128, 300, 257),
+    (2, 8, 1, 128, 128, 100), (1, 32, 8, 64, 768, 700), (2, 16, 8, 128, 520, 519), (1, 4, 4, 128, 16, 7),
+])
+def test_gqa_decode_attention(B, N, Kh, H, C, step):
+  T = G.Keep()
+  rng = np.random.default_rng(B * 1000 + C)
+  Lbuf = C
+  q = bf16_round(rng.standard_normal((B, 1, N, H)).astype(np.float32))
+  k = bf16_round(rng.standard_normal((B, C, Kh, H)).astype(np.float32))
+  v = bf16_round(rng.standard_normal((B, C, Kh, H)).astype(np.float32))
+  in_mask = np.ones((B, Lbuf), bool)
+  for b in range(B):  # left padding of different lengths plus a hole (a pad id inside a prompt)
+    in_mask[b, : (b * 5) % max(step, 1)] = False
+  if step > 3:
+    in_mask[0, step // 2] = False
+  in_mask[:, step] = True
+  lib = _lib.lib()
+  ws_bytes = lib.tmx_gqa_decode_workspace_bytes(B, N, Kh, H, C)
+  ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=G.DEV)
+  out = torch.empty(B, N * H, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_gqa_decode_attention', S(), T.bf(q), T.bf(k), T.bf(v), T.u8(in_mask),
+         T.i32([step]), Lbuf, G.p(out), G.p(ws), B, N, Kh, H, C)
+  G.sync()
+  from oracle import masks as OMK
+  mask = OMK.compute_attention_masks(step, C, ~in_mask)
+  fused = L.gqa_attention(q, k, v, mask, BF16, 'fused').reshape(B, -1)
+  ref = L.gqa_attention(q, k, v, mask, BF16, 'reference').reshape(B, -1)
+  got = G.host(out)
+  # kernel keeps f32 inside: 1 ulp against the f32-internal oracle, bf16 noise against the
+  # reference-rounding oracle (scores and probabilities rounded to bf16 there)
+  G.assert_bf16_close(got, fused, ulps=1.0, extra=1e-3, what='attention vs f32-internal oracle')
+  assert np.abs(got - ref).max() < 2e-2
+
+
+def _head_inputs(M, D, V, seed):
+  rng = np.random.default_rng(seed)
+  x = bf16_round(rng.standard_normal((M, D)).astype(np.float32))
+  w = bf16_round(rng.standard_normal((V, D)).astype(np.float32) * 0.05)
+  return x, w
+
+
+def _run_head(x, w, mode, temperature, key, step, forbidden=(), eos=(-1,), col_len=20):
+  T = G.Keep()
+  M, D = x.shape
+  V = w.shape[0]
+  lib = _lib.lib()
+  ws = torch.empty(lib.tmx_head_sample_workspace_bytes(M, V), dtype=torch.uint8, device=G.DEV)
+  tok = torch.full((M, col_len), -5, dtype=torch.int32, device=G.DEV)
+  lp = torch.zeros(M, col_len, dtype=torch.float32, device=G.DEV)
+  done = torch.zeros(M, dtype=torch.uint8, device=G.DEV)
+  logits = torch.empty(M, V, dtype=torch.float32, device=G.DEV)
+  fb = T.i32(list(forbidden)) if forbidden else None
+  G.call('tmx_head_sample', S(), T.bf(x), T.bf(w), M, D, V, mode, temperature, int(key[0]), int(key[1]),
+         T.i32([step]), fb, len(forbidden), T.i32(list(eos)), len(eos), G.p(tok), G.p(lp),
+         G.p(done), col_len, G.p(logits), G.p(ws))
+  G.sync()
+  return tok.cpu().numpy(), lp.cpu().numpy(), done.cpu().numpy(), logits.cpu().numpy()
+
+
+@pytest.mark.parametrize('M,D,V', [(1, 256, 1024), (5, 512, 4096), (64, 256, 1056), (100, 128, 2048)])
+def test_head_greedy(M, D, V):
+  T = G.Keep()
+  x, w = _head_inputs(M, D, V, M + V)
+  step = 3
+  tok, lp, done, logits = _run_head(x, w, 0, 1.0, (0, 0), step, eos=(int(0),))
+  ref_logits = bf16_round(x @ w.T)
+  G.assert_bf16_close(logits, ref_logits, ulps=1.0, min_exact=0.995, what='logits')
+  # selection and log-softmax are exact functions of the kernel's own logits
+  want_tok, want_lp = OS.sample_best(logits)
+  np.testing.assert_array_equal(tok[:, step + 1], want_tok)
+  np.testing.assert_allclose(lp[:, step + 1], want_lp, atol=2e-5)
+  assert np.all(tok[:, :step + 1] == -5) and np.all(tok[:, step + 2:] == -5)
+  np.testing.assert_array_equal(done, (want_tok == 0).astype(np.uint8))
+  # against the oracle's logits: same token wherever the top-2 margin exceeds the tolerance
+  o_tok, o_lp = OS.sample_best(ref_logits)
+  srt = np.sort(ref_logits, axis=-1)
+  clear = (srt[:, -1] - srt[:, -2]) > 2e-2
+  np.testing.assert_array_equal(tok[clear, step + 1], o_tok[clear])
+  assert clear.sum() == 0 or np.abs(lp[clear, step + 1] - o_lp[clear]).max() <= 1e-2
+
+
+def test_head_greedy_ties_pick_first_index_and_forbidden():
+  T = G.Keep()
+  M, D, V = 3, 128, 1024
+  x, w = _head_inputs(M, D, V, 5)
+  w[700] = w[13]
+  w[900] = w[13]
+  x[:] = bf16_round(w[13] * 4)[None, :]  # row 13 (and its copies) win by a wide margin
+  tok, lp, _, logits = _run_head(x, w, 0, 1.0, (0, 0), 0)
+  assert logits[0, 13] == logits[0, 700] == logits[0, 900] == logits[0].max()
+  assert np.all(tok[:, 1] == 13)
+  tok, _, _, _ = _run_head(x, w, 0, 1.0, (0, 0), 0, forbidden=(13,))
+  assert np.all(tok[:, 1] == 700)
+  tok, lp, _, _ = _run_head(x, w, 0, 1.0, (0, 0), 0, forbidden=(13, 700, 900, 5))
+  assert not np.isin(tok[:, 1], [13, 700, 900, 5]).any() and np.isfinite(lp[:, 1]).all()
+
+
+@pytest.mark.parametrize('M,D,V,temp', [(4, 256, 1024, 0.9), (64, 128, 4096, 1.0), (33, 256, 2080, 0.7)])
+def test_head_temperature_sampling_matches_threefry_oracle(M, D, V, temp):
+  T = G.Keep()
+  x, w = _head_inputs(M, D, V, V + 1)
+  seed_key = prng.prng_key(1234)
+  step = 6
+  tok, lp, _, logits = _run_head(x, w, 1, temp, seed_key, step)
+  z = (logits / np.float32(temp)).astype(np.float32)
+  key = prng.fold_in(seed_key, step)
+  noisy = z + prng.gumbel(key, z.shape)
+  want = np.argmax(noisy, axis=-1)
+  srt = np.sort(noisy, axis=-1)
+  clear = (srt[:, -1] - srt[:, -2]) > 1e-4  # GPU logf differs from numpy by an ulp or two
+  assert clear.mean() > 0.9
+  np.testing.assert_array_equal(tok[clear, step + 1], want[clear])
+  want_lp = OS.log_softmax(z)[np.arange(M), tok[:, step + 1]]
+  np.testing.assert_allclose(lp[:, step + 1], want_lp, atol=3e-5)
+  # a different step or seed gives a different draw
+  tok2, _, _, _ = _run_head(x, w, 1, temp, seed_key, step + 1)
+  tok3, _, _, _ = _run_head(x, w, 1, temp, prng.prng_key(99), step)
+  if M >= 16:
+    assert (tok2[:, step + 2] != tok[:, step + 1]).mean() > 0.5
+    assert (tok3[:, step + 1] != tok[:, step + 1]).mean() > 0.5
+
+
+def test_head_sampling_distribution_chi2():
+  T = G.Keep()
+  # one sharp row repeated: empirical frequencies follow softmax(z)
+  M, D, V = 128, 128, 1024
+  x, w = _head_inputs(1, D, V, 77)
+  w *= 8
+  x = np.repeat(x, M, axis=0)
+  counts = np.zeros(V)
+  for s in range(16):
+    tok, _, _, logits = _run_head(x, w, 1, 1.0, prng.prng_key(5), s)
+    counts += np.bincount(tok[:, s + 1], minlength=V)
+  pr = OS.softmax(logits[:1])[0].astype(np.float64)
+  top = np.argsort(-pr)[:8]
+  n = counts.sum()
+  obs = np.append(counts[top], n - counts[top].sum())
+  exp = np.append(pr[top], 1 - pr[top].sum()) * n
+  assert ((obs - exp) ** 2 / exp).sum() < 27.9  # 8 dof, p = 0.0005

@@ -6,7 +6,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, 'libtmx.so')
+LIB_PATH = os.environ.get('TMX_LIB', os.path.join(_HERE, 'libtmx.so'))
 
 _lib = None
 
@@ -17,19 +17,23 @@ SIGNATURES = {
     'tmx_abi_version': [],
     'tmx_int4_dequant': [vp, vp, vp, vp, ci, ci, ci],
     'tmx_qlora_linear': [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
+    'tmx_qlora_linear_num_splits': [ci, ci, ci],
+    'tmx_qlora_linear_planes': [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci],
     'tmx_rmsnorm': [vp, vp, vp, vp, ci, ci, cf, ci],
-    'tmx_lora_residual_rmsnorm': [vp, vp, vp, ci, vp, ci, cf, vp, vp, vp, vp, ci, ci, cf, ci],
-    'tmx_rope_kv_write': [vp, vp, vp, ci, vp, ci, cf, vp, vp, vp, vp, ci, vp, vp, vp, ci, ci, ci, ci, ci,
-                          cf, cf, ci],
-    'tmx_swiglu': [vp, vp, vp, ci, vp, ci, cf, vp, ci, ci],
+    'tmx_lora_residual_rmsnorm': [vp, vp, vp, ci, vp, ci, vp, ci, cf, vp, vp, vp, vp, ci, ci, cf, ci],
+    'tmx_rope_kv_write': [vp, vp, vp, ci, vp, ci, vp, ci, cf, vp, vp, vp, vp, ci, vp, vp, vp, ci, ci, ci,
+                          ci, ci, cf, cf, ci],
+    'tmx_swiglu': [vp, vp, vp, ci, vp, ci, vp, ci, cf, vp, ci, ci],
     'tmx_gqa_decode_attention': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci],
     'tmx_head_sample': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
                         vp, vp],
     'tmx_decode_steps': [vp, vp, vp, ci, ci],
+    'tmx_decode_steps_profiled': [vp, vp, vp, ci, ci, vp, vp],
 }
 # entry points that return size_t
 SIZE_FUNCS = {
     'tmx_gqa_decode_workspace_bytes': [ci, ci, ci, ci, ci],
+    'tmx_qlora_linear_workspace_bytes': [ci, ci, ci],
     'tmx_head_sample_workspace_bytes': [ci, ci],
     'tmx_decode_workspace_bytes': [vp, ci, ci],
 }

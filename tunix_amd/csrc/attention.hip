@@ -218,8 +218,10 @@ int gqa_decode(hipStream_t st, AttnArgs a, int H) {
 #define TMX_ATTN_CASE(HH, GG) \
   if (H == HH && G == GG) return launch_attn<HH, GG>(st, a);
   TMX_ATTN_CASE(64, 1)
+  TMX_ATTN_CASE(64, 2)
   TMX_ATTN_CASE(64, 4)
   TMX_ATTN_CASE(128, 1)
+  TMX_ATTN_CASE(128, 2)
   TMX_ATTN_CASE(128, 4)
   TMX_ATTN_CASE(128, 8)
 #undef TMX_ATTN_CASE

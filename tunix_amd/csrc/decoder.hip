@@ -8,6 +8,8 @@
 // live in device memory exactly like _SamplingState (sampler.py:53-109), and the
 // counter is advanced on the device, so the host never reads anything back
 // between steps.
+#include <vector>
+
 #include "tmx_kernels.h"
 
 namespace tmx {
@@ -15,11 +17,25 @@ namespace tmx {
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Workspace {
-  uint16_t *x, *xn, *qkv, *q, *attn, *yo, *gu, *act, *t;
+  uint16_t *x, *xn, *q, *attn, *act, *y16;
+  float *y_part, *t_part, *rope_tab;
   float* attn_partial;
   void* head_partial;
   size_t total;
 };
+
+struct Splits { int qkv, o, gate_up, down; };
+
+static Splits plan_splits(const tmx_model_desc* m, int B) {
+  const int D = m->embed_dim, NH = m->num_heads * m->head_dim;
+  const int QKV = NH + 2 * m->num_kv_heads * m->head_dim, F = m->hidden_dim;
+  Splits s;
+  s.qkv = qlinear_num_splits(D, QKV, B);
+  s.o = qlinear_num_splits(NH, D, B);
+  s.gate_up = qlinear_num_splits(D, 2 * F, B);
+  s.down = qlinear_num_splits(F, D, B);
+  return s;
+}
 
 static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   Workspace w;
@@ -27,25 +43,43 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   auto take = [&](size_t bytes) { char* p = base ? base + off : nullptr; off += align256(bytes); return p; };
   const size_t D = m->embed_dim, NH = (size_t)m->num_heads * m->head_dim;
   const size_t QKV = NH + 2 * (size_t)m->num_kv_heads * m->head_dim, F = m->hidden_dim;
+  const Splits sp = plan_splits(m, B);
+  size_t ypart = sp.qkv * QKV;
+  if (sp.o * D > ypart) ypart = sp.o * D;
+  if (sp.down * D > ypart) ypart = sp.down * D;
+  if (sp.gate_up > 1 && sp.gate_up * 2 * F > ypart) ypart = sp.gate_up * 2 * F;
   w.x = (uint16_t*)take(B * D * 2);
   w.xn = (uint16_t*)take(B * D * 2);
-  w.qkv = (uint16_t*)take(B * QKV * 2);
   w.q = (uint16_t*)take(B * NH * 2);
   w.attn = (uint16_t*)take(B * NH * 2);
-  w.yo = (uint16_t*)take(B * D * 2);
-  w.gu = (uint16_t*)take(B * 2 * F * 2);
   w.act = (uint16_t*)take(B * F * 2);
-  w.t = (uint16_t*)take((size_t)B * TMX_MAX_RPAD * 2);
+  w.y16 = (uint16_t*)take(B * 2 * F * 2);
+  w.y_part = (float*)take((size_t)B * ypart * 4);
+  w.t_part = (float*)take((size_t)TMX_MAX_SPLITS * B * TMX_MAX_RPAD * 4);
+  w.rope_tab = (float*)take((size_t)B * m->head_dim * 4);
   w.attn_partial = (float*)take(attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C));
   w.head_partial = take(head_partial_bytes(B, m->vocab_size));
   w.total = off;
   return w;
 }
 
+// Optional per-kernel-class timing with HIP events (used by the benchmark only).
+struct Prof {
+  std::vector<hipEvent_t> ev[TMX_NUM_KERNEL_CLASSES];
+  void before(int k, hipStream_t st) { push(k, st); }
+  void after(int k, hipStream_t st) { push(k, st); }
+  void push(int k, hipStream_t st) {
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    (void)hipEventRecord(e, st);
+    ev[k].push_back(e);
+  }
+};
+
 static int check_linear(const tmx_qlinear_desc& l, int K, int N) {
   if (!l.qweight || !l.scales) return TMX_ERR_ARG;
   if (l.K != K || l.N != N) return TMX_ERR_SHAPE;
-  if (l.lora_a_t && (!l.lora_b || l.rank <= 0 || l.r_pad > TMX_MAX_RPAD)) return TMX_ERR_ARG;
+  if (l.lora_a_t && (!l.lora_b || l.rank <= 0 || l.r_pad > TMX_MAX_RPAD || l.rank > 64)) return TMX_ERR_ARG;
   return TMX_OK;
 }
 
@@ -58,8 +92,8 @@ extern "C" size_t tmx_decode_workspace_bytes(const tmx_model_desc* m, int batch,
   return carve(m, batch, cache_size, nullptr).total;
 }
 
-extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
-                                int n_steps, int sample) {
+static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
+                             int n_steps, int sample, Prof* prof) {
   if (!m || !s || !m->layers || !m->embed || !m->final_norm_w || !m->head) return TMX_ERR_ARG;
   if (!s->token_buffer || !s->positions || !s->input_mask || !s->done || !s->step || !s->kv_cache ||
       !s->workspace)
@@ -85,42 +119,64 @@ extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state*
   const size_t kv_elems = (size_t)B * C * Kh * H;
   const float theta = m->family == TMX_FAMILY_LLAMA3 ? 1000000.0f : m->rope_theta;
   int rc;
-#define TMX_TRY(expr) \
-  if ((rc = (expr)) != TMX_OK) return rc;
+#define TMX_TRY(kind, expr)            \
+  {                                    \
+    if (prof) prof->before(kind, st);  \
+    rc = (expr);                       \
+    if (prof) prof->after(kind, st);   \
+    if (rc != TMX_OK) return rc;       \
+  }
 
+  const Splits sp = plan_splits(m, B);
+  auto lora_of = [&](const tmx_qlinear_desc& l, int nsplit) {
+    LoraIn li = {};
+    if (l.lora_a_t) {
+      li.t_part = w.t_part;
+      li.ldt = TMX_MAX_RPAD;
+      li.nsplit = nsplit;
+      li.b = (const uint16_t*)l.lora_b;
+      li.r = l.rank;
+      li.ls = l.lora_scale;
+    }
+    return li;
+  };
   for (int it = 0; it < n_steps; ++it) {
-    {  // embedding gather + first input norm
+    {  // embedding gather + first input norm + this step's RoPE table
       RowNormArgs a = {};
       a.embed = (const uint16_t*)m->embed;
       a.token_buffer = s->token_buffer;
       a.step = s->step;
       a.buf_len = L;
+      a.positions = s->positions;
+      a.rope_tab = w.rope_tab;
+      a.half = H / 2;
+      a.theta = theta;
       a.x_out = w.x;
       a.norm_w = (const uint16_t*)m->layers[0].norm1_w;
       a.xn_out = w.xn;
       a.D = D; a.eps = m->norm_eps; a.family = m->family;
-      TMX_TRY(row_norm(st, a, B));
+      TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
     }
     for (int i = 0; i < m->num_layers; ++i) {
       const tmx_layer_desc& l = m->layers[i];
       uint16_t* kc = (uint16_t*)s->kv_cache + (size_t)(2 * i) * kv_elems;
       uint16_t* vc = kc + kv_elems;
-      TMX_TRY(qlinear_base(st, w.xn, D, l.qkv.qweight, l.qkv.scales, l.qkv.lora_a_t, w.qkv, QKV, w.t,
-                           TMX_MAX_RPAD, B, D, QKV, l.qkv.G, l.qkv.r_pad));
+      TMX_TRY(TMX_K_QKV, qlinear_base(st, w.xn, D, l.qkv.qweight, l.qkv.scales, l.qkv.lora_a_t, nullptr,
+                                      w.y_part, w.t_part, TMX_MAX_RPAD, B, D, QKV, l.qkv.G, l.qkv.r_pad,
+                                      sp.qkv));
       {
         RopeArgs a = {};
-        a.qkv = w.qkv;
-        a.t = l.qkv.lora_a_t ? w.t : nullptr;
-        a.ldt = TMX_MAX_RPAD;
-        a.lora_b = (const uint16_t*)l.qkv.lora_b;
-        a.r = l.qkv.rank; a.ls = l.qkv.lora_scale;
+        a.qkv_part = w.y_part;
+        a.nsplit = sp.qkv;
+        a.lora = lora_of(l.qkv, sp.qkv);
         a.q_norm_w = (const uint16_t*)l.q_norm_w;
         a.k_norm_w = (const uint16_t*)l.k_norm_w;
         a.positions = s->positions; a.step = s->step; a.buf_len = L;
+        a.rope_tab = w.rope_tab;
         a.q_out = w.q; a.kcache = kc; a.vcache = vc;
         a.N = N; a.Kh = Kh; a.H = H; a.C = C;
         a.theta = theta; a.eps = m->norm_eps; a.family = m->family;
-        TMX_TRY(rope_kvwrite(st, a, B));
+        TMX_TRY(TMX_K_ROPE, rope_kvwrite(st, a, B));
       }
       {
         AttnArgs a = {};
@@ -129,48 +185,47 @@ extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state*
         a.out = w.attn; a.partial = w.attn_partial;
         a.B = B; a.N = N; a.Kh = Kh; a.C = C;
         a.scale = 1.0f / sqrtf((float)H);
-        TMX_TRY(gqa_decode(st, a, H));
+        TMX_TRY(TMX_K_ATTN, gqa_decode(st, a, H));
       }
-      TMX_TRY(qlinear_base(st, w.attn, NH, l.o.qweight, l.o.scales, l.o.lora_a_t, w.yo, D, w.t,
-                           TMX_MAX_RPAD, B, NH, D, l.o.G, l.o.r_pad));
+      TMX_TRY(TMX_K_O, qlinear_base(st, w.attn, NH, l.o.qweight, l.o.scales, l.o.lora_a_t, nullptr,
+                                    w.y_part, w.t_part, TMX_MAX_RPAD, B, NH, D, l.o.G, l.o.r_pad, sp.o));
       {
         RowNormArgs a = {};
-        a.y = w.yo;
-        a.t = l.o.lora_a_t ? w.t : nullptr;
-        a.ldt = TMX_MAX_RPAD;
-        a.lora_b = (const uint16_t*)l.o.lora_b;
-        a.r = l.o.rank; a.ls = l.o.lora_scale;
+        a.y_part = w.y_part;
+        a.nsplit = sp.o;
+        a.lora = lora_of(l.o, sp.o);
         a.residual = w.x; a.x_out = w.x;
         a.norm_w = (const uint16_t*)l.norm2_w; a.xn_out = w.xn;
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
-        TMX_TRY(row_norm(st, a, B));
+        TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
       }
-      TMX_TRY(qlinear_base(st, w.xn, D, l.gate_up.qweight, l.gate_up.scales, l.gate_up.lora_a_t, w.gu,
-                           2 * F, w.t, TMX_MAX_RPAD, B, D, 2 * F, l.gate_up.G, l.gate_up.r_pad));
+      const bool gu16 = sp.gate_up == 1;
+      TMX_TRY(TMX_K_GATE_UP, qlinear_base(st, w.xn, D, l.gate_up.qweight, l.gate_up.scales,
+                                          l.gate_up.lora_a_t, gu16 ? w.y16 : nullptr, w.y_part, w.t_part,
+                                          TMX_MAX_RPAD, B, D, 2 * F, l.gate_up.G, l.gate_up.r_pad,
+                                          sp.gate_up));
       {
         SwigluArgs a = {};
-        a.gu = w.gu;
-        a.t = l.gate_up.lora_a_t ? w.t : nullptr;
-        a.ldt = TMX_MAX_RPAD;
-        a.lora_b = (const uint16_t*)l.gate_up.lora_b;
-        a.r = l.gate_up.rank; a.ls = l.gate_up.lora_scale;
+        a.gu_bf16 = gu16 ? w.y16 : nullptr;
+        a.gu_part = w.y_part;
+        a.nsplit = sp.gate_up;
+        a.lora = lora_of(l.gate_up, sp.gate_up);
         a.act = w.act; a.F = F;
-        TMX_TRY(swiglu(st, a, B));
+        TMX_TRY(TMX_K_SWIGLU, swiglu(st, a, B));
       }
-      TMX_TRY(qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t, w.yo, D, w.t,
-                           TMX_MAX_RPAD, B, F, D, l.down.G, l.down.r_pad));
+      TMX_TRY(TMX_K_DOWN, qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t,
+                                       nullptr, w.y_part, w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G,
+                                       l.down.r_pad, sp.down));
       {
         RowNormArgs a = {};
-        a.y = w.yo;
-        a.t = l.down.lora_a_t ? w.t : nullptr;
-        a.ldt = TMX_MAX_RPAD;
-        a.lora_b = (const uint16_t*)l.down.lora_b;
-        a.r = l.down.rank; a.ls = l.down.lora_scale;
+        a.y_part = w.y_part;
+        a.nsplit = sp.down;
+        a.lora = lora_of(l.down, sp.down);
         a.residual = w.x; a.x_out = w.x;
         a.norm_w = (const uint16_t*)(i + 1 < m->num_layers ? m->layers[i + 1].norm1_w : m->final_norm_w);
         a.xn_out = w.xn;
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
-        TMX_TRY(row_norm(st, a, B));
+        TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
       }
     }
     if (sample) {
@@ -192,10 +247,35 @@ extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state*
       a.done = s->done;
       a.eos = s->eos_ids; a.n_eos = s->n_eos;
       a.buf_len = L;
-      TMX_TRY(head_sample(st, a));
+      TMX_TRY(TMX_K_HEAD, head_sample(st, a));
     }
-    TMX_TRY(advance_step(st, s->step));
+    TMX_TRY(TMX_K_ADVANCE, advance_step(st, s->step));
   }
 #undef TMX_TRY
   return TMX_OK;
+}
+
+extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
+                                int n_steps, int sample) {
+  return decode_steps_impl(m, s, stream, n_steps, sample, nullptr);
+}
+
+extern "C" int tmx_decode_steps_profiled(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
+                                         int n_steps, int sample, float* class_ms_host,
+                                         int* class_launches_host) {
+  if (!class_ms_host || !class_launches_host) return TMX_ERR_ARG;
+  Prof prof;
+  int rc = decode_steps_impl(m, s, stream, n_steps, sample, &prof);
+  (void)hipStreamSynchronize((hipStream_t)stream);
+  for (int k = 0; k < TMX_NUM_KERNEL_CLASSES; ++k) {
+    float total = 0.f;
+    for (size_t i = 0; i + 1 < prof.ev[k].size(); i += 2) {
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, prof.ev[k][i], prof.ev[k][i + 1]) == hipSuccess) total += ms;
+    }
+    class_ms_host[k] = total;
+    class_launches_host[k] = (int)(prof.ev[k].size() / 2);
+    for (hipEvent_t e : prof.ev[k]) (void)hipEventDestroy(e);
+  }
+  return rc;
 }

@@ -17,92 +17,179 @@
 
 namespace tmx {
 
-// delta for output column n of row m: bf16(bf16(sum_r t[r] * B[r][n]) * ls)
-__device__ __forceinline__ float lora_delta(const uint16_t* __restrict__ t_row,
-                                            const uint16_t* __restrict__ b, int ldb, int n, int r,
-                                            float ls) {
-  float d = 0.f;
-  for (int rr = 0; rr < r; ++rr) d = fmaf(bf2f(t_row[rr]), bf2f(b[(size_t)rr * ldb + n]), d);
-  return rbf(rbf(d) * ls);
+__device__ __forceinline__ void unpack8(const uint4& v, float* o) {
+  o[0] = bf_lo(v.x); o[1] = bf_hi(v.x); o[2] = bf_lo(v.y); o[3] = bf_hi(v.y);
+  o[4] = bf_lo(v.z); o[5] = bf_hi(v.z); o[6] = bf_lo(v.w); o[7] = bf_hi(v.w);
+}
+__device__ __forceinline__ uint4 pack8(const float* o) {
+  uint4 v;
+  v.x = pack_bf2(o[0], o[1]); v.y = pack_bf2(o[2], o[3]);
+  v.z = pack_bf2(o[4], o[5]); v.w = pack_bf2(o[6], o[7]);
+  return v;
 }
 
+// t_s[rr] = bf16(sum_s t_part[s][m][col0 + rr]) for rr < n, by the first n threads.
+__device__ __forceinline__ void stage_t(float* t_s, const LoraIn& l, int m, int M, int col0, int n) {
+  if ((int)threadIdx.x < n) {
+    float t = 0.f;
+    for (int s = 0; s < l.nsplit; ++s) t += l.t_part[((size_t)s * M + m) * l.ldt + col0 + threadIdx.x];
+    t_s[threadIdx.x] = rbf(t);
+  }
+}
+
+// 8 adjacent outputs n0..n0+7 of one row: base = bf16(sum of the split planes) or the bf16 tensor.
+__device__ __forceinline__ void load_base8(const uint16_t* y_bf16, const float* y_part, int nsplit, int m,
+                                           int M, int N, int n0, float* o) {
+  if (y_bf16) {
+    unpack8(*reinterpret_cast<const uint4*>(y_bf16 + (size_t)m * N + n0), o);
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float4* p = reinterpret_cast<const float4*>(y_part + ((size_t)s * M + m) * N + n0);
+    const float4 a = p[0], b = p[1];
+    o[0] += a.x; o[1] += a.y; o[2] += a.z; o[3] += a.w;
+    o[4] += b.x; o[5] += b.y; o[6] += b.z; o[7] += b.w;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = rbf(o[e]);
+}
+
+// o[e] = bf16(o[e] + bf16(bf16(sum_r t_s[r] B[r][n0 + e]) * ls))
+__device__ __forceinline__ void add_lora8(float* o, const float* t_s, const uint16_t* b, int ldb, int n0,
+                                          int r, float ls) {
+  float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int rr = 0; rr < r; ++rr) {
+    float w[8];
+    unpack8(*reinterpret_cast<const uint4*>(b + (size_t)rr * ldb + n0), w);
+    const float t = t_s[rr];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) d[e] = fmaf(t, w[e], d[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = rbf(o[e] + rbf(rbf(d[e]) * ls));
+}
 
 // One workgroup per row: h = bf16(bf16(y + delta) + residual); xn = RMSNorm(h).
-template <int EPT>  // elements per thread, D <= 256 * EPT
+// In embedding mode it also fills this step's RoPE sin/cos table row.
+template <int CPT>  // 8-element chunks per thread, D <= 2048 * CPT
 __global__ __launch_bounds__(256) void row_norm_kernel(RowNormArgs a) {
   __shared__ float smem[8];
-  const int m = blockIdx.x;
-  float v[EPT];
+  __shared__ float t_s[TMX_MAX_RPAD];
+  const int m = blockIdx.x, M = gridDim.x;
+  float v[CPT][8];
   float ss = 0.f;
   const uint16_t* src = nullptr;
   if (a.embed) {
-    const int tok = a.token_buffer[(size_t)m * a.buf_len + *a.step];
+    const int step = *a.step;
+    const int tok = a.token_buffer[(size_t)m * a.buf_len + step];
     src = a.embed + (size_t)tok * a.D;
-  }
-#pragma unroll
-  for (int e = 0; e < EPT; ++e) {
-    const int n = e * 256 + threadIdx.x;
-    float x = 0.f;
-    if (n < a.D) {
-      if (src) {
-        x = bf2f(src[n]);
-      } else {
-        x = bf2f(a.y[(size_t)m * a.D + n]);
-        if (a.t) x = rbf(x + lora_delta(a.t + (size_t)m * a.ldt, a.lora_b, a.D, n, a.r, a.ls));
-        if (a.residual) x = rbf(x + bf2f(a.residual[(size_t)m * a.D + n]));
-      }
-      if (a.x_out) a.x_out[(size_t)m * a.D + n] = f2bf(x);
+    if (a.rope_tab && (int)threadIdx.x < a.half) {
+      const float pos = (float)a.positions[(size_t)m * a.buf_len + step];
+      const float frac = 2.f * (float)threadIdx.x / (float)(2 * a.half);
+      const float ang = pos / powf(a.theta, frac);
+      a.rope_tab[((size_t)m * a.half + threadIdx.x) * 2] = sinf(ang);
+      a.rope_tab[((size_t)m * a.half + threadIdx.x) * 2 + 1] = cosf(ang);
     }
-    v[e] = x;
-    ss += x * x;
+  } else if (a.lora.t_part) {
+    stage_t(t_s, a.lora, m, M, 0, a.lora.r);
+    __syncthreads();
+  }
+  const int nchunks = a.D >> 3;
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
+    if (c < nchunks) {
+      const int n0 = c * 8;
+      if (src) {
+        unpack8(*reinterpret_cast<const uint4*>(src + n0), v[i]);
+      } else {
+        load_base8(a.y_bf16, a.y_part, a.nsplit, m, M, a.D, n0, v[i]);
+        if (a.lora.t_part) add_lora8(v[i], t_s, a.lora.b, a.D, n0, a.lora.r, a.lora.ls);
+        if (a.residual) {
+          float r8[8];
+          unpack8(*reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0), r8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e] + r8[e]);
+        }
+      }
+      if (a.x_out) *reinterpret_cast<uint4*>(a.x_out + (size_t)m * a.D + n0) = pack8(v[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+    }
   }
   if (!a.norm_w) return;
   ss = block_sum<4>(ss, smem);
   const float rms = sqrtf(ss / (float)a.D + a.eps);
 #pragma unroll
-  for (int e = 0; e < EPT; ++e) {
-    const int n = e * 256 + threadIdx.x;
-    if (n < a.D) {
-      const float w = bf2f(a.norm_w[n]);
-      float o;
-      if (a.family == TMX_FAMILY_LLAMA3) o = rbf(w * v[e]) / rms;
-      else o = w * (v[e] / rms);
-      a.xn_out[(size_t)m * a.D + n] = f2bf(o);
+  for (int i = 0; i < CPT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nchunks) {
+      const int n0 = c * 8;
+      float w[8], o[8];
+      unpack8(*reinterpret_cast<const uint4*>(a.norm_w + n0), w);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (a.family == TMX_FAMILY_LLAMA3) o[e] = rbf(w[e] * v[i][e]) / rms;
+        else o[e] = w[e] * (v[i][e] / rms);
+      }
+      *reinterpret_cast<uint4*>(a.xn_out + (size_t)m * a.D + n0) = pack8(o);
     }
   }
 }
 
 int row_norm(hipStream_t st, const RowNormArgs& a, int M) {
-  if (a.D <= 0 || a.D > 256 * 32) return TMX_ERR_SHAPE;
-  const int ept = (a.D + 255) / 256;
-  if (ept <= 1) hipLaunchKernelGGL(row_norm_kernel<1>, dim3(M), dim3(256), 0, st, a);
-  else if (ept <= 4) hipLaunchKernelGGL(row_norm_kernel<4>, dim3(M), dim3(256), 0, st, a);
-  else if (ept <= 8) hipLaunchKernelGGL(row_norm_kernel<8>, dim3(M), dim3(256), 0, st, a);
-  else if (ept <= 16) hipLaunchKernelGGL(row_norm_kernel<16>, dim3(M), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(row_norm_kernel<32>, dim3(M), dim3(256), 0, st, a);
+  if (a.D <= 0 || a.D % 8 || a.D > 2048 * 8) return TMX_ERR_SHAPE;
+  if (a.lora.t_part && a.lora.r > TMX_MAX_RPAD) return TMX_ERR_SHAPE;
+  if (a.rope_tab && a.half > 256) return TMX_ERR_SHAPE;
+  const int cpt = (a.D / 8 + 255) / 256;
+  if (cpt <= 1) hipLaunchKernelGGL(row_norm_kernel<1>, dim3(M), dim3(256), 0, st, a);
+  else if (cpt <= 2) hipLaunchKernelGGL(row_norm_kernel<2>, dim3(M), dim3(256), 0, st, a);
+  else if (cpt <= 4) hipLaunchKernelGGL(row_norm_kernel<4>, dim3(M), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(row_norm_kernel<8>, dim3(M), dim3(256), 0, st, a);
   return check_launch();
 }
 
 // ---------------------------------------------------------------------------
-
 // grid (N + 2 Kh, B), one wave per head vector; lane i owns elements i and i + H/2.
 __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
-  const int head = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  __shared__ float t_s[64];
+  const int head = blockIdx.x, b = blockIdx.y, B = gridDim.y, lane = threadIdx.x;
   const int half = a.H >> 1;
   const int step = *a.step;
   const bool active = lane < half;
   const int ntot = (a.N + 2 * a.Kh) * a.H;
   const int kind = head < a.N ? 0 : (head < a.N + a.Kh ? 1 : 2);  // q, k, v
   const int col0 = head * a.H;
+  if (a.lora.t_part) {
+    stage_t(t_s, a.lora, b, B, kind * a.lora.r, a.lora.r);
+    __syncthreads();
+  }
   float x1 = 0.f, x2 = 0.f;
   if (active) {
-    const size_t base = (size_t)b * ntot + col0;
-    x1 = bf2f(a.qkv[base + lane]);
-    x2 = bf2f(a.qkv[base + lane + half]);
-    if (a.t) {
-      const uint16_t* trow = a.t + (size_t)b * a.ldt + kind * a.r;
-      x1 = rbf(x1 + lora_delta(trow, a.lora_b, ntot, col0 + lane, a.r, a.ls));
-      x2 = rbf(x2 + lora_delta(trow, a.lora_b, ntot, col0 + lane + half, a.r, a.ls));
+    const int c1 = col0 + lane, c2 = c1 + half;
+    if (a.qkv_bf16) {
+      x1 = bf2f(a.qkv_bf16[(size_t)b * ntot + c1]);
+      x2 = bf2f(a.qkv_bf16[(size_t)b * ntot + c2]);
+    } else {
+      for (int s = 0; s < a.nsplit; ++s) {
+        x1 += a.qkv_part[((size_t)s * B + b) * ntot + c1];
+        x2 += a.qkv_part[((size_t)s * B + b) * ntot + c2];
+      }
+      x1 = rbf(x1);
+      x2 = rbf(x2);
+    }
+    if (a.lora.t_part) {
+      float d1 = 0.f, d2 = 0.f;
+      for (int rr = 0; rr < a.lora.r; ++rr) {
+        d1 = fmaf(t_s[rr], bf2f(a.lora.b[(size_t)rr * ntot + c1]), d1);
+        d2 = fmaf(t_s[rr], bf2f(a.lora.b[(size_t)rr * ntot + c2]), d2);
+      }
+      x1 = rbf(x1 + rbf(rbf(d1) * a.lora.ls));
+      x2 = rbf(x2 + rbf(rbf(d2) * a.lora.ls));
     }
   }
   const int slot = step % a.C;
@@ -123,13 +210,18 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
       x2 = rbf(bf2f(nw[lane + half]) * (x2 / rms));
     }
   }
-  float o1 = 0.f, o2 = 0.f;
   if (active) {
-    const float pos = (float)a.positions[(size_t)b * a.buf_len + step];
-    const float frac = 2.f * (float)lane / (float)a.H;
-    const float timescale = powf(a.theta, frac);
-    const float ang = pos / timescale;
-    float sn = sinf(ang), cs = cosf(ang);
+    float sn, cs;
+    if (a.rope_tab) {
+      sn = a.rope_tab[((size_t)b * half + lane) * 2];
+      cs = a.rope_tab[((size_t)b * half + lane) * 2 + 1];
+    } else {
+      const float pos = (float)a.positions[(size_t)b * a.buf_len + step];
+      const float ang = pos / powf(a.theta, 2.f * (float)lane / (float)a.H);
+      sn = sinf(ang);
+      cs = cosf(ang);
+    }
+    float o1, o2;
     if (a.family == TMX_FAMILY_LLAMA3) {
       o1 = x1 * cs - x2 * sn;
       o2 = x2 * cs + x1 * sn;
@@ -149,28 +241,40 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
 
 int rope_kvwrite(hipStream_t st, const RopeArgs& a, int B) {
   if (a.H > 128 || a.H % 2) return TMX_ERR_SHAPE;
+  if (a.lora.t_part && a.lora.r > 64) return TMX_ERR_SHAPE;
   hipLaunchKernelGGL(rope_kvwrite_kernel, dim3(a.N + 2 * a.Kh, B), dim3(64), 0, st, a);
   return check_launch();
 }
 
 // ---------------------------------------------------------------------------
-
+// grid (ceil(F / 2048), M): a thread owns 8 adjacent hidden units of one row.
 __global__ __launch_bounds__(256) void swiglu_kernel(SwigluArgs a) {
-  const int f = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
-  if (f >= a.F) return;
-  float g = bf2f(a.gu[(size_t)m * 2 * a.F + f]);
-  float u = bf2f(a.gu[(size_t)m * 2 * a.F + a.F + f]);
-  if (a.t) {
-    const uint16_t* trow = a.t + (size_t)m * a.ldt;
-    g = rbf(g + lora_delta(trow, a.lora_b, 2 * a.F, f, a.r, a.ls));
-    u = rbf(u + lora_delta(trow + a.r, a.lora_b, 2 * a.F, a.F + f, a.r, a.ls));
+  __shared__ float t_s[TMX_MAX_RPAD];
+  const int m = blockIdx.y, M = gridDim.y;
+  if (a.lora.t_part) {
+    stage_t(t_s, a.lora, m, M, 0, 2 * a.lora.r);
+    __syncthreads();
   }
-  const float sg = rbf(1.f / (1.f + expf(-g)));
-  a.act[(size_t)m * a.F + f] = f2bf(rbf(g * sg) * u);
+  const int f0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (f0 >= a.F) return;
+  float g[8], u[8], o[8];
+  load_base8(a.gu_bf16, a.gu_part, a.nsplit, m, M, 2 * a.F, f0, g);
+  load_base8(a.gu_bf16, a.gu_part, a.nsplit, m, M, 2 * a.F, a.F + f0, u);
+  if (a.lora.t_part) {
+    add_lora8(g, t_s, a.lora.b, 2 * a.F, f0, a.lora.r, a.lora.ls);
+    add_lora8(u, t_s + a.lora.r, a.lora.b, 2 * a.F, a.F + f0, a.lora.r, a.lora.ls);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float sg = rbf(1.f / (1.f + expf(-g[e])));
+    o[e] = rbf(g[e] * sg) * u[e];
+  }
+  *reinterpret_cast<uint4*>(a.act + (size_t)m * a.F + f0) = pack8(o);
 }
 
 int swiglu(hipStream_t st, const SwigluArgs& a, int M) {
-  hipLaunchKernelGGL(swiglu_kernel, dim3((a.F + 255) / 256, M), dim3(256), 0, st, a);
+  if (a.F % 8 || (a.lora.t_part && 2 * a.lora.r > TMX_MAX_RPAD)) return TMX_ERR_SHAPE;
+  hipLaunchKernelGGL(swiglu_kernel, dim3((a.F + 2047) / 2048, M), dim3(256), 0, st, a);
   return check_launch();
 }
 
@@ -187,12 +291,23 @@ int advance_step(hipStream_t st, int32_t* step) {
 
 using namespace tmx;
 
+static LoraIn make_lora(const void* t_part, int ldt, int nsplit, const void* b, int r, float ls) {
+  LoraIn l = {};
+  l.t_part = (const float*)t_part;
+  l.ldt = ldt;
+  l.nsplit = nsplit;
+  l.b = (const uint16_t*)b;
+  l.r = r;
+  l.ls = ls;
+  return l;
+}
+
 extern "C" int tmx_rmsnorm(void* stream, const void* x, const void* w, void* y, int M, int D, float eps,
                            int family) {
   if (!x || !w || !y) return TMX_ERR_ARG;
   if (M <= 0) return TMX_ERR_SHAPE;
   RowNormArgs a = {};
-  a.y = (const uint16_t*)x;
+  a.y_bf16 = (const uint16_t*)x;
   a.norm_w = (const uint16_t*)w;
   a.xn_out = (uint16_t*)y;
   a.D = D;
@@ -201,19 +316,18 @@ extern "C" int tmx_rmsnorm(void* stream, const void* x, const void* w, void* y, 
   return row_norm((hipStream_t)stream, a, M);
 }
 
-extern "C" int tmx_lora_residual_rmsnorm(void* stream, const void* y, const void* t, int ldt,
-                                         const void* lora_b, int r, float lora_scale,
-                                         const void* residual, void* x_out, const void* norm_w,
-                                         void* xn_out, int M, int D, float eps, int family) {
-  if (!y || (t && !lora_b) || (norm_w && !xn_out)) return TMX_ERR_ARG;
-  if (M <= 0) return TMX_ERR_SHAPE;
+extern "C" int tmx_lora_residual_rmsnorm(void* stream, const void* y_bf16, const float* y_part,
+                                         int nsplit, const float* t_part, int ldt, const void* lora_b,
+                                         int r, float lora_scale, const void* residual, void* x_out,
+                                         const void* norm_w, void* xn_out, int M, int D, float eps,
+                                         int family) {
+  if ((!y_bf16 && !y_part) || (t_part && !lora_b) || (norm_w && !xn_out)) return TMX_ERR_ARG;
+  if (M <= 0 || (!y_bf16 && nsplit < 1)) return TMX_ERR_SHAPE;
   RowNormArgs a = {};
-  a.y = (const uint16_t*)y;
-  a.t = (const uint16_t*)t;
-  a.ldt = ldt;
-  a.lora_b = (const uint16_t*)lora_b;
-  a.r = r;
-  a.ls = lora_scale;
+  a.y_bf16 = (const uint16_t*)y_bf16;
+  a.y_part = y_part;
+  a.nsplit = nsplit;
+  a.lora = make_lora(t_part, ldt, nsplit, lora_b, r, lora_scale);
   a.residual = (const uint16_t*)residual;
   a.x_out = (uint16_t*)x_out;
   a.norm_w = (const uint16_t*)norm_w;
@@ -224,20 +338,21 @@ extern "C" int tmx_lora_residual_rmsnorm(void* stream, const void* y, const void
   return row_norm((hipStream_t)stream, a, M);
 }
 
-extern "C" int tmx_rope_kv_write(void* stream, const void* qkv, const void* t, int ldt,
-                                 const void* lora_b, int r, float lora_scale, const void* q_norm_w,
-                                 const void* k_norm_w, const int32_t* positions, const int32_t* step,
-                                 int buf_len, void* q_out, void* kcache, void* vcache, int B, int N,
-                                 int Kh, int H, int C, float theta, float eps, int family) {
-  if (!qkv || !positions || !step || !q_out || !kcache || !vcache || (t && !lora_b)) return TMX_ERR_ARG;
-  if (B <= 0 || N <= 0 || Kh <= 0 || C <= 0) return TMX_ERR_SHAPE;
+extern "C" int tmx_rope_kv_write(void* stream, const void* qkv_bf16, const float* qkv_part, int nsplit,
+                                 const float* t_part, int ldt, const void* lora_b, int r,
+                                 float lora_scale, const void* q_norm_w, const void* k_norm_w,
+                                 const int32_t* positions, const int32_t* step, int buf_len, void* q_out,
+                                 void* kcache, void* vcache, int B, int N, int Kh, int H, int C,
+                                 float theta, float eps, int family) {
+  if ((!qkv_bf16 && !qkv_part) || !positions || !step || !q_out || !kcache || !vcache ||
+      (t_part && !lora_b))
+    return TMX_ERR_ARG;
+  if (B <= 0 || N <= 0 || Kh <= 0 || C <= 0 || (!qkv_bf16 && nsplit < 1)) return TMX_ERR_SHAPE;
   RopeArgs a = {};
-  a.qkv = (const uint16_t*)qkv;
-  a.t = (const uint16_t*)t;
-  a.ldt = ldt;
-  a.lora_b = (const uint16_t*)lora_b;
-  a.r = r;
-  a.ls = lora_scale;
+  a.qkv_bf16 = (const uint16_t*)qkv_bf16;
+  a.qkv_part = qkv_part;
+  a.nsplit = nsplit;
+  a.lora = make_lora(t_part, ldt, nsplit, lora_b, r, lora_scale);
   a.q_norm_w = (const uint16_t*)q_norm_w;
   a.k_norm_w = (const uint16_t*)k_norm_w;
   a.positions = positions;
@@ -251,17 +366,16 @@ extern "C" int tmx_rope_kv_write(void* stream, const void* qkv, const void* t, i
   return rope_kvwrite((hipStream_t)stream, a, B);
 }
 
-extern "C" int tmx_swiglu(void* stream, const void* gate_up, const void* t, int ldt, const void* lora_b,
-                          int r, float lora_scale, void* act, int M, int F) {
-  if (!gate_up || !act || (t && !lora_b)) return TMX_ERR_ARG;
-  if (M <= 0 || F <= 0) return TMX_ERR_SHAPE;
+extern "C" int tmx_swiglu(void* stream, const void* gate_up_bf16, const float* gate_up_part, int nsplit,
+                          const float* t_part, int ldt, const void* lora_b, int r, float lora_scale,
+                          void* act, int M, int F) {
+  if ((!gate_up_bf16 && !gate_up_part) || !act || (t_part && !lora_b)) return TMX_ERR_ARG;
+  if (M <= 0 || F <= 0 || (!gate_up_bf16 && nsplit < 1)) return TMX_ERR_SHAPE;
   SwigluArgs a = {};
-  a.gu = (const uint16_t*)gate_up;
-  a.t = (const uint16_t*)t;
-  a.ldt = ldt;
-  a.lora_b = (const uint16_t*)lora_b;
-  a.r = r;
-  a.ls = lora_scale;
+  a.gu_bf16 = (const uint16_t*)gate_up_bf16;
+  a.gu_part = gate_up_part;
+  a.nsplit = nsplit;
+  a.lora = make_lora(t_part, ldt, nsplit, lora_b, r, lora_scale);
   a.act = (uint16_t*)act;
   a.F = F;
   return swiglu((hipStream_t)stream, a, M);

@@ -19,8 +19,11 @@ namespace tmx {
 // Expand one 32-bit word (8 nibbles, element j = 2 (i % 4) + i / 4 for nibble i)
 // into the 8 bf16 B-operand values of one MFMA step: bf16((u - 8) * s).
 __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s) {
-  const uint32_t lo = d & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
-  const uint32_t hi = (d >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7 in bytes 0..3
+  uint32_t lo = d & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
+  uint32_t hi = (d >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7 in bytes 0..3
+  // keep the two masked words opaque so that each byte is widened by one
+  // v_cvt_f32_ubyteN instead of a bit-field extract plus a conversion
+  asm volatile("" : "+v"(lo), "+v"(hi));
   // nibble i: byte i/2 of (i even ? lo : hi)
   const float n0 = (float)(lo & 0xFF), n1 = (float)(hi & 0xFF);
   const float n2 = (float)((lo >> 8) & 0xFF), n3 = (float)((hi >> 8) & 0xFF);
@@ -38,151 +41,280 @@ __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s)
 }
 
 
-// One workgroup = 4 waves owns NSUB adjacent 32-column tiles over the whole K;
-// the waves take k-tiles round-robin (their loads form one contiguous 4 KiB
-// stream per column tile) and the partial accumulators meet in LDS.
-template <int MT, int NSUB>
-__global__ __launch_bounds__(256) void qlinear_mfma_kernel(QLinearArgs a) {
-  extern __shared__ float red[];  // [4][NSUB*MT*16][64]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// One workgroup = 4 waves owns a block of 4 * NSUB adjacent 32-column tiles (one
+// group of NSUB tiles per wave) over one K-slice.  The activation k-tile
+// x[0:M, 64 kb : 64 kb + 64] is fetched once per workgroup with coalesced 16-byte
+// loads, double-buffered in LDS (rows padded to 144 bytes: conflict-free
+// ds_read_b128) and shared by the four waves as MFMA A fragments; weights go
+// HBM -> registers.  Global loads of k-tile i+1 are issued before the MFMAs of
+// k-tile i.  Small-N projections are split along K over blockIdx.y so that
+// every CU streams weights; each split writes its own f32 plane (summed by the
+// consumer kernel), so results do not depend on scheduling order.
+constexpr int kXStride = 72;  // bf16 elements per LDS row (64 + 8 pad)
+
+template <int V>
+struct IC { static constexpr int value = V; };
+
+// LORA = false: NSUB int4 column tiles per wave.  LORA = true: the block computes
+// t = x . A from dense bf16 columns of A^T [Rpad, K] (one 32-column tile per wave).
+template <int MT, int NSUB, bool LORA>
+__device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[MT * 32][kXStride]) {
+  // xs: 2 LDS buffers, buffer b holds activation tile i with i % 2 == b
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = lane >> 5, nl = lane & 31;
   const int KT = a.K >> 6;
-  const bool lora_block = (int)blockIdx.x >= a.n_main_blocks;
-  constexpr int NS = NSUB;
+  const int split = blockIdx.y;
+  const int kb0 = split * a.kt_per_split;
+  const int kb1 = (kb0 + a.kt_per_split < KT) ? kb0 + a.kt_per_split : KT;
+  const int kpg_shift = (a.G == 64) ? 0 : __builtin_ctz(a.G >> 6), KG = a.K / a.G;
 
-  f32x16_t acc[NS][MT];
+  // this wave's column tiles; waves past the last tile recompute the last one (their
+  // results are dropped) so that the pipelined loop below stays free of branches
+  const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
+  const int nb_first = LORA ? wave : ((int)blockIdx.x * 4 + wave) * NSUB;
+  int nbs[NSUB];
+  bool sub_ok[NSUB];
 #pragma unroll
-  for (int s = 0; s < NS; ++s)
+  for (int s = 0; s < NSUB; ++s) {
+    sub_ok[s] = (nb_first + s) < NT;
+    nbs[s] = sub_ok[s] ? nb_first + s : NT - 1;
+  }
+
+  f32x16_t acc[NSUB][MT];
+#pragma unroll
+  for (int s = 0; s < NSUB; ++s)
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[s][m][r] = 0.f;
 
-  const uint16_t* xrow[MT];
+  // cooperative activation load: chunk c = tid + 256 i -> row c / 8, 16-byte column c % 8
+  const uint16_t* xsrc[MT];
+  int xrow_l[MT], xcol_l[MT];
 #pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    int row = m * 32 + nl;
-    row = row < a.M ? row : a.M - 1;
-    xrow[m] = a.x + (size_t)row * a.ldx + h * 8;
+  for (int i = 0; i < MT; ++i) {
+    const int c = tid + 256 * i;
+    xrow_l[i] = c >> 3;
+    xcol_l[i] = (c & 7) * 8;
+    const int row = xrow_l[i] < a.M ? xrow_l[i] : a.M - 1;
+    xsrc[i] = a.x + (size_t)row * a.ldx + xcol_l[i];
   }
-
-  if (!lora_block) {
-    const int nb0 = blockIdx.x * NS;
-    const int kpg = a.G >> 6;  // k-tiles per scale group
-    const int KG = a.K / a.G;
-#pragma unroll 2
-    for (int kb = wave; kb < KT; kb += 4) {
-      uint4 w[NS];
-      float s[NS];
+  const u32x4_t* wsrc[NSUB];
+  const uint16_t* ssrc[NSUB];
 #pragma unroll
-      for (int sub = 0; sub < NS; ++sub) {
-        w[sub] = a.qw[((size_t)(nb0 + sub) * KT + kb) * 64 + lane];
-        s[sub] = bf2f(a.scales[((size_t)(nb0 + sub) * KG + kb / kpg) * 32 + nl]);
-      }
-      bf16x8_t xa[MT][4];
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-          xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xrow[m] + kb * 64 + t * 16);
-#pragma unroll
-      for (int sub = 0; sub < NS; ++sub) {
-        const float m8s = -8.f * s[sub];
-        const uint32_t wd[4] = {w[sub].x, w[sub].y, w[sub].z, w[sub].w};
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const bf16x8_t b = dequant_word(wd[t], s[sub], m8s);
-#pragma unroll
-          for (int m = 0; m < MT; ++m)
-            acc[sub][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[sub][m], 0, 0, 0);
-        }
-      }
-    }
-  } else {
-    // LoRA A tile: dense bf16 columns c of A^T [Rpad, K]; only sub-tile 0 is used.
-    const int ct = blockIdx.x - a.n_main_blocks;
-    const uint16_t* arow = a.a_t + (size_t)(ct * 32 + nl) * a.K + h * 8;
-#pragma unroll 2
-    for (int kb = wave; kb < KT; kb += 4) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(arow + kb * 64 + t * 16);
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-          const bf16x8_t xv = *reinterpret_cast<const bf16x8_t*>(xrow[m] + kb * 64 + t * 16);
-          acc[0][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xv, b, acc[0][m], 0, 0, 0);
-        }
-      }
+  for (int s = 0; s < NSUB; ++s) {
+    if (LORA) {
+      wsrc[s] = reinterpret_cast<const u32x4_t*>(a.a_t + (size_t)(nbs[s] * 32 + nl) * a.K + h * 8);
+      ssrc[s] = nullptr;
+    } else {
+      wsrc[s] = reinterpret_cast<const u32x4_t*>(a.qw) + (size_t)nbs[s] * KT * 64 + lane;
+      ssrc[s] = a.scales + (size_t)nbs[s] * KG * 32 + nl;
     }
   }
 
-  // Cross-wave reduction through LDS, then a coalesced bf16 store.
-  constexpr int NIDX = NS * MT * 16;
+  constexpr int P = 4;               // tiles in flight per wave (HBM latency >> one k-tile of math)
+  constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
+  u32x4_t xring[P][MT];
+  u32x4_t wring[P][NSUB][WPT];
+  uint16_t sring[P][NSUB];
+  const int nk = kb1 - kb0;
+  if (nk <= 0) return;
+  const int klast = kb1 - 1;
+
+  // Unconditional loads with clamped tile indices: the compiler can then count the
+  // outstanding loads exactly and wait only for the oldest one.
+  auto load_w = [&](int kb, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+    kb = kb < klast ? kb : klast;
+#ifdef TMX_DEBUG_SAME_TILE
+    kb = kb0;
+#endif
 #pragma unroll
-  for (int sub = 0; sub < NS; ++sub)
+    for (int s = 0; s < NSUB; ++s) {
+      if (LORA) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) wring[p][s][t] = wsrc[s][(size_t)kb * 8 + t * 2];
+      } else {
+#ifdef TMX_DEBUG_NO_WLOAD
+        wring[p][s][0] = u32x4_t{(uint32_t)kb, 0x12345678u, (uint32_t)lane, 0x9abcdef0u};
+        sring[p][s] = 0x3c00;
+#else
+        wring[p][s][0] = wsrc[s][(size_t)kb * 64];
+#ifdef TMX_DEBUG_NO_SLOAD
+        sring[p][s] = 0x3c00;
+#else
+        sring[p][s] = ssrc[s][(size_t)(kb >> kpg_shift) * 32];
+#endif
+#endif
+      }
+    }
+  };
+  auto load_x = [&](int kb, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+    kb = kb < klast ? kb : klast;
+#ifdef TMX_DEBUG_SAME_X
+    kb = kb0;
+#endif
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xring[p][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + kb * 64);
+  };
+  auto stash_x = [&](int buf, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      *reinterpret_cast<u32x4_t*>(&xs[buf][xrow_l[i]][xcol_l[i]]) = xring[p][i];
+  };
+  // one k-tile (tile kb, ring slot p, LDS buffer p & 1): read the A fragments, consume and
+  // refill the weight slot, do the math, publish activation tile kb + 1 to the other buffer
+  auto tile_step = [&](int kb, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+    constexpr int p1 = (p + 1) % P;
+    bf16x8_t xa[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        red[((size_t)wave * NIDX + (sub * MT + m) * 16 + r) * 64 + lane] = acc[sub][m][r];
-  __syncthreads();
-  const int nsub_used = lora_block ? 1 : NS;
-  for (int e = threadIdx.x; e < NIDX * 64; e += 256) {
-    const int idx = e >> 6, ln = e & 63;
-    const int sub = idx / (MT * 16), m = (idx / 16) % MT, r = idx & 15;
-    if (sub >= nsub_used) continue;
-    const float v = red[(size_t)idx * 64 + ln] + red[((size_t)NIDX + idx) * 64 + ln] +
-                    red[((size_t)2 * NIDX + idx) * 64 + ln] + red[((size_t)3 * NIDX + idx) * 64 + ln];
-    const int row = m * 32 + acc_row(r, ln);
-    if (row >= a.M) continue;
-    if (!lora_block) {
-      const int col = (blockIdx.x * NS + sub) * 32 + (ln & 31);
-      a.y[(size_t)row * a.ldy + col] = f2bf(v);
-    } else {
-      const int col = (blockIdx.x - a.n_main_blocks) * 32 + (ln & 31);
-      a.t[(size_t)row * a.ldt + col] = f2bf(v);
+      for (int t = 0; t < 4; ++t)
+        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(&xs[p & 1][m * 32 + nl][t * 16 + h * 8]);
+    u32x4_t wc[NSUB][WPT];
+    float s_c[NSUB];
+#pragma unroll
+    for (int s = 0; s < NSUB; ++s) {
+#pragma unroll
+      for (int t = 0; t < WPT; ++t) wc[s][t] = wring[p][s][t];
+      s_c[s] = LORA ? 0.f : bf2f(sring[p][s]);
     }
+    load_w(kb + P, pc);
+#pragma unroll
+    for (int s = 0; s < NSUB; ++s) {
+      const float m8s = -8.f * s_c[s];
+      const uint32_t wd[4] = {wc[s][0].x, wc[s][0].y, wc[s][0].z, wc[s][0].w};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        bf16x8_t b;
+        if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[s][t % WPT]);
+#ifdef TMX_DEBUG_NO_DEQUANT
+        else b = __builtin_bit_cast(bf16x8_t, wc[s][0]);
+#else
+        else b = dequant_word(wd[t], s_c[s], m8s);
+#endif
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#ifdef TMX_DEBUG_NO_MFMA
+          acc[s][m][t] += __builtin_bit_cast(f32x4_t, b)[0] * __builtin_bit_cast(f32x4_t, xa[m][t])[1];
+#else
+          acc[s][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[s][m], 0, 0, 0);
+#endif
+      }
+    }
+#ifndef TMX_DEBUG_NO_STASH
+    stash_x((p + 1) & 1, IC<p1>{});
+    load_x(kb + 1 + P, IC<p1>{});
+    __syncthreads();
+#endif
+  };
+
+  // prologue: P activation tiles and P weight tiles in flight, tile 0 published
+  load_x(kb0 + 0, IC<0>{}); load_x(kb0 + 1, IC<1>{}); load_x(kb0 + 2, IC<2>{}); load_x(kb0 + 3, IC<3>{});
+  load_w(kb0 + 0, IC<0>{}); load_w(kb0 + 1, IC<1>{}); load_w(kb0 + 2, IC<2>{}); load_w(kb0 + 3, IC<3>{});
+  stash_x(0, IC<0>{});
+  load_x(kb0 + P, IC<0>{});
+  __syncthreads();
+  const int ngroups = nk / P;
+  for (int g = 0; g < ngroups; ++g) {
+    const int kb = kb0 + g * P;
+    tile_step(kb + 0, IC<0>{});
+    tile_step(kb + 1, IC<1>{});
+    tile_step(kb + 2, IC<2>{});
+    tile_step(kb + 3, IC<3>{});
+  }
+  {
+    const int kb = kb0 + ngroups * P;
+    const int rem = nk - ngroups * P;
+    if (rem > 0) tile_step(kb + 0, IC<0>{});
+    if (rem > 1) tile_step(kb + 1, IC<1>{});
+    if (rem > 2) tile_step(kb + 2, IC<2>{});
+  }
+
+  // epilogue: every wave owns its tiles outright
+#pragma unroll
+  for (int s = 0; s < NSUB; ++s) {
+    if (!sub_ok[s]) continue;
+    const int col = (nb_first + s) * 32 + nl;
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m * 32 + acc_row(r, lane);
+        if (row >= a.M) continue;
+        if (LORA) a.t_part[((size_t)split * a.M + row) * a.ldt + col] = acc[s][m][r];
+        else if (a.y_bf16) a.y_bf16[(size_t)row * a.N + col] = f2bf(acc[s][m][r]);
+        else a.y_part[((size_t)split * a.M + row) * a.N + col] = acc[s][m][r];
+      }
   }
 }
 
 template <int MT, int NSUB>
+__global__ __launch_bounds__(256, 2) void qlinear_mfma_kernel(QLinearArgs a) {
+  __shared__ __align__(16) uint16_t xs[2][MT * 32][kXStride];
+  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block<MT, 1, true>(a, xs);
+  else gemm_block<MT, NSUB, false>(a, xs);
+}
+
+template <int MT, int NSUB>
 static int launch_qlinear(hipStream_t st, QLinearArgs a) {
-  a.n_main_blocks = a.N / (32 * NSUB);
-  const int blocks = a.n_main_blocks + (a.a_t ? a.Rpad / 32 : 0);
-  const size_t lds = (size_t)4 * NSUB * MT * 16 * 64 * sizeof(float);
-  hipLaunchKernelGGL((qlinear_mfma_kernel<MT, NSUB>), dim3(blocks), dim3(256), lds, st, a);
+  const int cols_per_block = 128 * NSUB;
+  a.n_main_blocks = (a.N + cols_per_block - 1) / cols_per_block;
+  const int blocks = a.n_main_blocks + (a.a_t ? 1 : 0);
+  hipLaunchKernelGGL((qlinear_mfma_kernel<MT, NSUB>), dim3(blocks, a.nsplit), dim3(256), 0, st, a);
   return check_launch();
 }
 
+// Number of K-slices for a projection: enough workgroups to cover the chip, at
+// least 4 k-tiles per slice.
+int qlinear_num_splits(int K, int N, int M) {
+  const int nsub = (N >= 16384 && M <= 64) ? 2 : 1;
+  const int nblocks = (N + 128 * nsub - 1) / (128 * nsub);
+  const int KT = K / 64;
+  int s = (256 + nblocks - 1) / nblocks;
+  const int smax = KT / 4 > 0 ? KT / 4 : 1;
+  if (s > smax) s = smax;
+  if (s > TMX_MAX_SPLITS) s = TMX_MAX_SPLITS;
+  if (s < 1) s = 1;
+  // slices are whole groups of 4 k-tiles; drop slices that would be empty
+  const int per = ((KT + s - 1) / s + 3) / 4 * 4;
+  return (KT + per - 1) / per;
+}
+
 // Host-side dispatch shared by the C entry point and the decode-step launcher.
+// Output: y_bf16 [M, N] when nsplit == 1 and y_bf16 != null, else y_part
+// [nsplit][M][N] f32 planes.  t_part: [nsplit][M][ldt] f32 (LoRA projection).
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
-                 const void* a_t, void* y, int ldy, void* t, int ldt, int M, int K, int N, int G,
-                 int Rpad) {
-  if (!x || !qw || !scales || !y) return TMX_ERR_ARG;
-  if (M <= 0 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
-  if (K % 64 || N % 32 || G % 64 || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
-  if (a_t && (!t || Rpad <= 0 || Rpad % 32)) return TMX_ERR_SHAPE;
-  for (int m0 = 0; m0 < M; m0 += 128) {
-    const int mc = (M - m0) < 128 ? (M - m0) : 128;
-    QLinearArgs a;
-    a.x = (const uint16_t*)x + (size_t)m0 * ldx;
-    a.ldx = ldx;
-    a.qw = (const uint4*)qw;
-    a.scales = (const uint16_t*)scales;
-    a.a_t = (const uint16_t*)a_t;
-    a.y = (uint16_t*)y + (size_t)m0 * ldy;
-    a.ldy = ldy;
-    a.t = t ? (uint16_t*)t + (size_t)m0 * ldt : nullptr;
-    a.ldt = ldt;
-    a.M = mc; a.K = K; a.N = N; a.G = G; a.Rpad = Rpad;
-    int rc;
-    const bool wide = (N % 64 == 0) && (N / 64 >= 384);
-    if (mc <= 32) rc = wide ? launch_qlinear<1, 2>(st, a) : launch_qlinear<1, 1>(st, a);
-    else if (mc <= 64) rc = wide ? launch_qlinear<2, 2>(st, a) : launch_qlinear<2, 1>(st, a);
-    else rc = launch_qlinear<4, 1>(st, a);
-    if (rc != TMX_OK) return rc;
-  }
-  return TMX_OK;
+                 const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
+                 int N, int G, int Rpad, int nsplit) {
+  if (!x || !qw || !scales || (!y_bf16 && !y_part)) return TMX_ERR_ARG;
+  if (M <= 0 || M > 128 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
+  if (K % 64 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
+  if (a_t && (!t_part || Rpad <= 0 || Rpad % 32 || Rpad > 128 || ldt < Rpad)) return TMX_ERR_SHAPE;
+  if (nsplit < 1 || (nsplit > 1 && !y_part)) return TMX_ERR_ARG;
+  QLinearArgs a;
+  a.x = (const uint16_t*)x;
+  a.ldx = ldx;
+  a.qw = (const uint4*)qw;
+  a.scales = (const uint16_t*)scales;
+  a.a_t = (const uint16_t*)a_t;
+  a.y_bf16 = (nsplit == 1) ? (uint16_t*)y_bf16 : nullptr;
+  a.y_part = y_part;
+  a.t_part = t_part;
+  a.ldt = ldt;
+  a.M = M; a.K = K; a.N = N; a.G = G; a.Rpad = Rpad;
+  a.nsplit = nsplit;
+  const int KT = K / 64;
+  a.kt_per_split = ((KT + nsplit - 1) / nsplit + 3) / 4 * 4;
+  if ((KT + a.kt_per_split - 1) / a.kt_per_split != nsplit) return TMX_ERR_SHAPE;  // empty slice
+  const bool wide = (N >= 16384);
+  if (M <= 32) return wide ? launch_qlinear<1, 2>(st, a) : launch_qlinear<1, 1>(st, a);
+  if (M <= 64) return wide ? launch_qlinear<2, 2>(st, a) : launch_qlinear<2, 1>(st, a);
+  return launch_qlinear<4, 1>(st, a);
 }
 
 // ---------------------------------------------------------------------------
@@ -212,22 +344,30 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(const uint4* qw, cons
   }
 }
 
-// y[m][n] <- bf16( y + bf16( bf16(sum_r t[m][r] B[r][n]) * ls ) ) (+ residual).
-// Rounding points follow the reference's bf16 einsum -> scale -> add chain.
-__global__ __launch_bounds__(256) void lora_apply_kernel(uint16_t* y, int ldy, const uint16_t* t,
-                                                         int ldt, const uint16_t* b, int r, float ls,
-                                                         const uint16_t* res, int ldres, int M, int N) {
+// y[m][n] = bf16( bf16(sum_s y_part[s][m][n]) + bf16( bf16(sum_r t[m][r] B[r][n]) * ls ) )
+// (+ residual), t[m][r] = bf16(sum_s t_part[s][m][r]).  Rounding points follow the
+// reference's bf16 einsum -> scale -> add chain.
+__global__ __launch_bounds__(256) void lora_apply_kernel(uint16_t* y, const float* y_part, int nsplit,
+                                                         const float* t_part, int ldt, const uint16_t* b,
+                                                         int r, float ls, const uint16_t* res, int M,
+                                                         int N) {
   const int n = blockIdx.x * 256 + threadIdx.x;
   const int m = blockIdx.y;
   if (n >= N) return;
-  float v = bf2f(y[(size_t)m * ldy + n]);
-  if (t) {
+  float v = 0.f;
+  for (int s = 0; s < nsplit; ++s) v += y_part[((size_t)s * M + m) * N + n];
+  v = rbf(v);
+  if (t_part) {
     float d = 0.f;
-    for (int rr = 0; rr < r; ++rr) d = fmaf(bf2f(t[(size_t)m * ldt + rr]), bf2f(b[(size_t)rr * N + n]), d);
+    for (int rr = 0; rr < r; ++rr) {
+      float t = 0.f;
+      for (int s = 0; s < nsplit; ++s) t += t_part[((size_t)s * M + m) * ldt + rr];
+      d = fmaf(rbf(t), bf2f(b[(size_t)rr * N + n]), d);
+    }
     v = rbf(v + rbf(rbf(d) * ls));
   }
-  if (res) v = rbf(v + bf2f(res[(size_t)m * ldres + n]));
-  y[(size_t)m * ldy + n] = f2bf(v);
+  if (res) v = rbf(v + bf2f(res[(size_t)m * N + n]));
+  y[(size_t)m * N + n] = f2bf(v);
 }
 
 }  // namespace tmx
@@ -244,21 +384,37 @@ extern "C" int tmx_int4_dequant(void* stream, const void* qweight, const void* s
   return check_launch();
 }
 
+extern "C" size_t tmx_qlora_linear_workspace_bytes(int M, int K, int N) {
+  const size_t s = qlinear_num_splits(K, N, M);
+  return s * (size_t)M * ((size_t)N + TMX_MAX_RPAD) * sizeof(float);
+}
+
+extern "C" int tmx_qlora_linear_num_splits(int M, int K, int N) { return qlinear_num_splits(K, N, M); }
+
+extern "C" int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight,
+                                       const void* scales, const void* lora_a_t, float* y_part,
+                                       float* t_part, int M, int K, int N, int G, int r_pad, int nsplit) {
+  return qlinear_base((hipStream_t)stream, x, K, qweight, scales, lora_a_t, nullptr, y_part, t_part,
+                      TMX_MAX_RPAD, M, K, N, G, r_pad, nsplit);
+}
+
 extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const void* scales,
                                 const void* lora_a_t, const void* lora_b, const void* residual,
-                                void* y, void* t_ws, int M, int K, int N, int G, int r, int r_pad,
+                                void* y, void* workspace, int M, int K, int N, int G, int r, int r_pad,
                                 float lora_scale) {
   hipStream_t st = (hipStream_t)stream;
   const bool lora = lora_a_t != nullptr;
-  if (lora && (!lora_b || !t_ws || r <= 0 || r > r_pad)) return TMX_ERR_ARG;
-  int rc = qlinear_base(st, x, K, qweight, scales, lora ? lora_a_t : nullptr, y, N, t_ws, r_pad, M, K, N,
-                        G, r_pad);
+  if (!workspace || !y) return TMX_ERR_ARG;
+  if (lora && (!lora_b || r <= 0 || r > r_pad)) return TMX_ERR_ARG;
+  if (M <= 0 || M > 128) return TMX_ERR_SHAPE;
+  const int ns = qlinear_num_splits(K, N, M);
+  float* y_part = (float*)workspace;
+  float* t_part = y_part + (size_t)ns * M * N;
+  int rc = qlinear_base(st, x, K, qweight, scales, lora ? lora_a_t : nullptr, nullptr, y_part, t_part,
+                        TMX_MAX_RPAD, M, K, N, G, r_pad, ns);
   if (rc != TMX_OK) return rc;
-  if (lora || residual) {
-    hipLaunchKernelGGL(lora_apply_kernel, dim3((N + 255) / 256, M), dim3(256), 0, st, (uint16_t*)y, N,
-                       lora ? (const uint16_t*)t_ws : nullptr, r_pad, (const uint16_t*)lora_b, r,
-                       lora_scale, (const uint16_t*)residual, N, M, N);
-    rc = check_launch();
-  }
-  return rc;
+  hipLaunchKernelGGL(lora_apply_kernel, dim3((N + 255) / 256, M), dim3(256), 0, st, (uint16_t*)y, y_part,
+                     ns, lora ? t_part : nullptr, TMX_MAX_RPAD, (const uint16_t*)lora_b, r, lora_scale,
+                     (const uint16_t*)residual, M, N);
+  return check_launch();
 }

@@ -5,31 +5,42 @@
 namespace tmx {
 
 struct QLinearArgs {
-  const uint16_t* x;       // [M, K] bf16
+  const uint16_t* x;       // [M, K] bf16 row-major
   int ldx;
   const uint4* qw;         // packed int4 tiles
   const uint16_t* scales;  // [N/32][K/G][32] bf16
   const uint16_t* a_t;     // LoRA A transposed [Rpad, K] bf16 (may be null)
-  uint16_t* y;             // [M, N] bf16 base output
-  int ldy;
-  uint16_t* t;             // [M, Rpad] bf16 LoRA projection output
+  uint16_t* y_bf16;        // [M, N] bf16 (only when nsplit == 1), else null
+  float* y_part;           // [nsplit][M][N] f32 planes
+  float* t_part;           // [nsplit][M][ldt] f32 LoRA projection planes
   int ldt;
   int M, K, N, G, Rpad;
-  int n_main_blocks;
+  int n_main_blocks, nsplit, kt_per_split;
+};
+
+// The LoRA-B half applied by the consumer of a projection.
+struct LoraIn {
+  const float* t_part;  // [nsplit][M][ldt] f32 planes of x . A (null: no LoRA)
+  int ldt, nsplit;
+  const uint16_t* b;    // [r][N] bf16
+  int r;
+  float ls;             // alpha / rank
 };
 
 struct RowNormArgs {
-  // source of the row: either an embedding gather (embed != null) or y (+ LoRA) (+ residual)
+  // source of the row: an embedding gather (embed != null) or y (+ LoRA) (+ residual)
   const uint16_t* embed;        // [V, D]
   const int32_t* token_buffer;  // [B, L]
   const int32_t* step;          // device scalar: column of token_buffer to read
   int buf_len;
-  const uint16_t* y;            // [M, D] base projection output
-  const uint16_t* t;            // [M, ldt] LoRA projection (null: none)
-  int ldt;
-  const uint16_t* lora_b;       // [r, D]
-  int r;
-  float ls;
+  const int32_t* positions;     // [B, L] (embedding mode: fills rope_tab)
+  float* rope_tab;              // [B][half][2] sin, cos of this step (may be null)
+  int half;
+  float theta;
+  const uint16_t* y_bf16;       // [M, D] base projection output, or
+  const float* y_part;          // [nsplit][M][D] f32 planes
+  int nsplit;
+  LoraIn lora;
   const uint16_t* residual;     // [M, D] (null: none)
   uint16_t* x_out;              // [M, D] new residual stream (null: not stored)
   const uint16_t* norm_w;       // [D] (null: no norm output)
@@ -40,19 +51,18 @@ struct RowNormArgs {
 };
 
 struct RopeArgs {
-  const uint16_t* qkv;   // [B, (N + 2 Kh) * H] base projection output
-  const uint16_t* t;     // [B, ldt]: x.A_q | x.A_k | x.A_v (null: no LoRA)
-  int ldt;
-  const uint16_t* lora_b;  // [r, (N + 2 Kh) * H]
-  int r;
-  float ls;
+  const uint16_t* qkv_bf16;  // [B, (N + 2 Kh) * H], or
+  const float* qkv_part;     // [nsplit][B][(N + 2 Kh) * H]
+  int nsplit;
+  LoraIn lora;               // t columns: x.A_q | x.A_k | x.A_v
   const uint16_t* q_norm_w;  // [H] (Qwen3) or null
   const uint16_t* k_norm_w;
   const int32_t* positions;  // [B, L]
   const int32_t* step;
   int buf_len;
-  uint16_t* q_out;   // [B, N * H]
-  uint16_t* kcache;  // [B, C, Kh, H]
+  const float* rope_tab;     // [B][H/2][2] or null (then sin/cos are computed here)
+  uint16_t* q_out;           // [B, N * H]
+  uint16_t* kcache;          // [B, C, Kh, H]
   uint16_t* vcache;
   int N, Kh, H, C;
   float theta, eps;
@@ -60,13 +70,11 @@ struct RopeArgs {
 };
 
 struct SwigluArgs {
-  const uint16_t* gu;  // [M, 2F]: gate columns then up columns
-  const uint16_t* t;   // [M, ldt]: x.A_gate | x.A_up
-  int ldt;
-  const uint16_t* lora_b;  // [r, 2F]
-  int r;
-  float ls;
-  uint16_t* act;  // [M, F]
+  const uint16_t* gu_bf16;  // [M, 2F]: gate columns then up columns, or
+  const float* gu_part;     // [nsplit][M][2F]
+  int nsplit;
+  LoraIn lora;              // t columns: x.A_gate | x.A_up
+  uint16_t* act;            // [M, F]
   int F;
 };
 
@@ -115,8 +123,9 @@ int gqa_decode(hipStream_t st, AttnArgs a, int H);
 size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
 int head_sample(hipStream_t st, HeadArgs a);
 size_t head_partial_bytes(int M, int V);
+int qlinear_num_splits(int K, int N, int M);
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
-                 const void* a_t, void* y, int ldy, void* t, int ldt, int M, int K, int N, int G,
-                 int Rpad);
+                 const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
+                 int N, int G, int Rpad, int nsplit);
 
 }  // namespace tmx

@@ -269,7 +269,9 @@ class QLoRAModel:
                        f' {sorted(cur.keys())[:3]}... vs {sorted(state.keys())[:3]}...')
     for k, v in state.items():
       v = torch.as_tensor(v)
-      if v.reshape(cur[k].shape[0], -1).shape != cur[k].shape and v.reshape(-1, cur[k].shape[-1]).shape != cur[k].shape:
+      ok = v.numel() == cur[k].numel() and (
+          v.reshape(cur[k].shape[0], -1).shape == cur[k].shape or v.reshape(-1, cur[k].shape[-1]).shape == cur[k].shape)
+      if not ok:
         raise ValueError('New state must have the same shape, dtype and sharding as the old state.'
                          f' {k}: {tuple(v.shape)} vs {tuple(cur[k].shape)}')
     for i, layer in enumerate(self.layers):
