@@ -44,6 +44,7 @@ extern "C" {
 
 #define TMX_MAX_RPAD 128   /* widest padded LoRA projection (sum of fused ranks, rounded up to 32) */
 #define TMX_MAX_SPLITS 16  /* most K-slices a projection is split into */
+#define TMX_MAX_LORA_SPLITS 32 /* most K-slices of the LoRA projection x . A */
 
 #define TMX_SAMPLE_GREEDY 0
 #define TMX_SAMPLE_TOP_P 1
@@ -60,7 +61,9 @@ int tmx_int4_dequant(void* stream, const void* qweight, const void* scales, void
 /* y[M, N] = bf16(x[M, K] . dequant(qweight)) (+ LoRA delta) (+ residual), M <= 128.
  * Replaces the qwix-wrapped Einsum / nnx.Linear call: tunix/models/llama3/model.py:216-218,
  * :489-496; tunix/models/qwen3/model.py:389-393, :1199-1208.
- *   lora_a_t : A transposed and zero-padded, bf16 [r_pad, K], r_pad % 32 == 0 (NULL: no LoRA)
+ *   lora_a_t : A in MFMA fragment order, bf16 [K/64][r_pad/32][64][4][8], r_pad % 32 == 0,
+ *              columns >= r zero (NULL: no LoRA): element A[64 kb + 16 t + 8 h + j][32 ct + c]
+ *              at ((((kb * (r_pad/32) + ct) * 64 + 32 h + c) * 4 + t) * 8 + j)
  *   lora_b   : bf16 [r, N]
  *   residual : bf16 [M, N] or NULL; added after the LoRA delta, in bf16
  *   workspace: tmx_qlora_linear_workspace_bytes(M, K, N) bytes (f32 K-slice planes) */
@@ -71,9 +74,11 @@ int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const voi
 
 /* The matrix product alone, for callers that fuse their own consumer: writes `nsplit` f32
  * K-slice planes y_part[nsplit][M][N] (their sum is x . dequant(W)) and, with LoRA,
- * t_part[nsplit][M][TMX_MAX_RPAD] (their sum is x . A).  nsplit in [1, TMX_MAX_SPLITS];
+ * t_part[tmx_qlora_linear_num_lora_splits(K)][M][TMX_MAX_RPAD] (their sum is x . A).
+ * nsplit in [1, TMX_MAX_SPLITS] and such that no K-slice is empty;
  * tmx_qlora_linear_num_splits() returns the count the library itself would pick. */
 int tmx_qlora_linear_num_splits(int M, int K, int N);
+int tmx_qlora_linear_num_lora_splits(int K);
 int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight, const void* scales,
                             const void* lora_a_t, float* y_part, float* t_part, int M, int K, int N,
                             int G, int r_pad, int nsplit);
@@ -89,13 +94,14 @@ int tmx_rmsnorm(void* stream, const void* x, const void* w, void* y, int M, int 
  * (*_bf16) or as `nsplit` f32 K-slice planes [nsplit][M][N] (*_part) that they sum and round
  * to bf16 first, and apply the LoRA-B half:
  *   delta[m, n] = bf16(bf16(sum_r t[m, r] lora_b[r, n]) * lora_scale),
- *   t[m, r] = bf16(sum_s t_part[s][m][r]), t_part f32 [nsplit][M][ldt] (NULL: no LoRA). */
+ *   t[m, r] = bf16(sum_s t_part[s][m][r]), t_part f32 [t_nsplit][M][ldt] (NULL: no LoRA). */
 
 /* h = bf16(bf16(y + delta) + residual) -> x_out;  xn_out = RMSNorm(h) * norm_w.
  * residual, x_out, norm_w may be NULL.  Residual wiring of
  * tunix/models/llama3/model.py:546-564, tunix/models/qwen3/model.py:1268-1289. */
 int tmx_lora_residual_rmsnorm(void* stream, const void* y_bf16, const float* y_part, int nsplit,
-                              const float* t_part, int ldt, const void* lora_b, int r, float lora_scale,
+                              const float* t_part, int t_nsplit, int ldt, const void* lora_b, int r,
+                              float lora_scale,
                               const void* residual, void* x_out, const void* norm_w, void* xn_out, int M,
                               int D, float eps, int family);
 
@@ -104,7 +110,8 @@ int tmx_lora_residual_rmsnorm(void* stream, const void* y_bf16, const float* y_p
  * K / V rows of cache slot *step % C.  tunix/models/llama3/model.py:249-270, :348-377;
  * tunix/models/qwen3/model.py:432-453, :559-597. */
 int tmx_rope_kv_write(void* stream, const void* qkv_bf16, const float* qkv_part, int nsplit,
-                      const float* t_part, int ldt, const void* lora_b, int r, float lora_scale,
+                      const float* t_part, int t_nsplit, int ldt, const void* lora_b, int r,
+                      float lora_scale,
                       const void* q_norm_w, const void* k_norm_w, const int32_t* positions,
                       const int32_t* step, int buf_len, void* q_out, void* kcache, void* vcache, int B,
                       int N, int Kh, int H, int C, float theta, float eps, int family);
@@ -112,8 +119,8 @@ int tmx_rope_kv_write(void* stream, const void* qkv_bf16, const float* qkv_part,
 /* act[M, F] = bf16(silu(gate) * up), gate_up[M, 2F] = gate columns then up columns
  * (+ deltas, t columns x.A_gate | x.A_up).  tunix/models/llama3/model.py:489-496. */
 int tmx_swiglu(void* stream, const void* gate_up_bf16, const float* gate_up_part, int nsplit,
-               const float* t_part, int ldt, const void* lora_b, int r, float lora_scale, void* act,
-               int M, int F);
+               const float* t_part, int t_nsplit, int ldt, const void* lora_b, int r, float lora_scale,
+               void* act, int M, int F);
 
 /* ---- GQA decode attention -------------------------------------------------- */
 
@@ -148,7 +155,7 @@ int tmx_head_sample(void* stream, const void* x, const void* head_w, int M, int 
 typedef struct {
   const void* qweight;  /* q4t tiles of the (column-fused) weight [K, N] */
   const void* scales;   /* bf16 [N/32][K/G][32] */
-  const void* lora_a_t; /* bf16 [r_pad, K]: fused A matrices side by side, transposed; NULL = no LoRA */
+  const void* lora_a_t; /* fused A matrices side by side in fragment order (see tmx_qlora_linear); NULL = no LoRA */
   const void* lora_b;   /* bf16 [rank, N]: B matrices side by side */
   int K, N, G, rank, r_pad;
   float lora_scale;     /* alpha / rank */

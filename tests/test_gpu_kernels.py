@@ -96,6 +96,7 @@ def test_qlora_linear_planes_sum_and_rejects():
   assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, 129, K, N, group, 0, 1) == -2  # M > 128
   assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, M, K, N, 96, 0, 1) == -2      # G not a power of two
   assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, M, K, N, group, 0, 3) == -2   # empty K-slice
+  assert lib.tmx_qlora_linear_num_lora_splits(4096) == 16 and lib.tmx_qlora_linear_num_lora_splits(14336) == 28
 
 
 @pytest.mark.parametrize('family', [0, 1])
@@ -118,13 +119,13 @@ def test_lora_residual_rmsnorm_planes(family):
   rng = np.random.default_rng(3)
   M, D, r, ns = 9, 1024, 16, 3
   yp = rng.standard_normal((ns, M, D)).astype(np.float32)
-  tp = rng.standard_normal((ns, M, 128)).astype(np.float32)
+  tp = rng.standard_normal((5, M, 128)).astype(np.float32)  # 5 LoRA planes: the generic sum
   b = bf16_round(rng.standard_normal((r, D)).astype(np.float32) * 0.05)
   res = bf16_round(rng.standard_normal((M, D)).astype(np.float32))
   w = bf16_round(rng.uniform(0.5, 1.5, D).astype(np.float32))
   x_out = torch.empty(M, D, dtype=torch.bfloat16, device=G.DEV)
   xn = torch.empty(M, D, dtype=torch.bfloat16, device=G.DEV)
-  G.call('tmx_lora_residual_rmsnorm', S(), None, T.f32(yp), ns, T.f32(tp), 128, T.bf(b), r, 1.5,
+  G.call('tmx_lora_residual_rmsnorm', S(), None, T.f32(yp), ns, T.f32(tp), 5, 128, T.bf(b), r, 1.5,
          T.bf(res), G.p(x_out), T.bf(w), G.p(xn), M, D, 1e-6, family)
   G.sync()
   y = bf16_round(yp.sum(0))
@@ -144,7 +145,7 @@ def test_rope_kv_write(family, H, N, Kh):
   B, C, Lbuf, r, ns, step = 3, 12, 10, 8, 2, 5
   ntot = (N + 2 * Kh) * H
   qkv = rng.standard_normal((ns, B, ntot)).astype(np.float32)
-  tp = rng.standard_normal((ns, B, 128)).astype(np.float32)
+  tp = rng.standard_normal((16, B, 128)).astype(np.float32)
   lb = bf16_round(rng.standard_normal((r, ntot)).astype(np.float32) * 0.05)
   qn = bf16_round(rng.uniform(0.5, 1.5, H).astype(np.float32))
   kn = bf16_round(rng.uniform(0.5, 1.5, H).astype(np.float32))
@@ -153,7 +154,7 @@ def test_rope_kv_write(family, H, N, Kh):
   vc = torch.full((B, C, Kh, H), 7.0, dtype=torch.bfloat16, device=G.DEV)
   q_out = torch.empty(B, N * H, dtype=torch.bfloat16, device=G.DEV)
   theta = 1_000_000.0 if family == 0 else 10_000.0
-  G.call('tmx_rope_kv_write', S(), None, T.f32(qkv), ns, T.f32(tp), 128, T.bf(lb), r, 2.0,
+  G.call('tmx_rope_kv_write', S(), None, T.f32(qkv), ns, T.f32(tp), 16, 128, T.bf(lb), r, 2.0,
          T.bf(qn) if family else None, T.bf(kn) if family else None, T.i32(positions),
          T.i32([step]), Lbuf, G.p(q_out), G.p(kc), G.p(vc), B, N, Kh, H, C, theta, 1e-6, family)
   G.sync()
@@ -192,12 +193,12 @@ def test_swiglu(M, F, ns):
   act = torch.empty(M, F, dtype=torch.bfloat16, device=G.DEV)
   if ns == 0:
     gu = bf16_round(rng.standard_normal((M, 2 * F)).astype(np.float32) * 2)
-    G.call('tmx_swiglu', S(), T.bf(gu), None, 0, None, 0, None, 0, 0.0, G.p(act), M, F)
+    G.call('tmx_swiglu', S(), T.bf(gu), None, 0, None, 0, 0, None, 0, 0.0, G.p(act), M, F)
     y = gu
   else:
     gp = rng.standard_normal((ns, M, 2 * F)).astype(np.float32)
-    tp = rng.standard_normal((ns, M, 128)).astype(np.float32)
-    G.call('tmx_swiglu', S(), None, T.f32(gp), ns, T.f32(tp), 128, T.bf(lb), r, 2.0, G.p(act), M, F)
+    tp = rng.standard_normal((28, M, 128)).astype(np.float32)
+    G.call('tmx_swiglu', S(), None, T.f32(gp), ns, T.f32(tp), 28, 128, T.bf(lb), r, 2.0, G.p(act), M, F)
     y = bf16_round(gp.sum(0))
     t = bf16_round(tp.sum(0))
     dg = bf16_round(bf16_round(t[:, :r] @ lb[:, :F]) * np.float32(2.0))

@@ -55,7 +55,7 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   w.act = (uint16_t*)take(B * F * 2);
   w.y16 = (uint16_t*)take(B * 2 * F * 2);
   w.y_part = (float*)take((size_t)B * ypart * 4);
-  w.t_part = (float*)take((size_t)TMX_MAX_SPLITS * B * TMX_MAX_RPAD * 4);
+  w.t_part = (float*)take((size_t)TMX_MAX_LORA_SPLITS * B * TMX_MAX_RPAD * 4);
   w.rope_tab = (float*)take((size_t)B * m->head_dim * 4);
   w.attn_partial = (float*)take(attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C));
   w.head_partial = take(head_partial_bytes(B, m->vocab_size));
@@ -128,12 +128,12 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   }
 
   const Splits sp = plan_splits(m, B);
-  auto lora_of = [&](const tmx_qlinear_desc& l, int nsplit) {
+  auto lora_of = [&](const tmx_qlinear_desc& l, int) {
     LoraIn li = {};
     if (l.lora_a_t) {
       li.t_part = w.t_part;
       li.ldt = TMX_MAX_RPAD;
-      li.nsplit = nsplit;
+      li.nsplit = qlinear_num_lora_splits(l.K);
       li.b = (const uint16_t*)l.lora_b;
       li.r = l.rank;
       li.ls = l.lora_scale;

@@ -28,13 +28,64 @@ __device__ __forceinline__ uint4 pack8(const float* o) {
   return v;
 }
 
+// Sums NS K-slice planes of 8 adjacent f32 values; all 2 * NS loads are issued before the
+// first add so that the planes' memory latencies overlap.  Planes are added in ascending
+// order whatever NS is, so every code path rounds identically.
+template <int NS>
+__device__ __forceinline__ void sum_planes8(const float* p, size_t stride, float* o) {
+  float4 a[NS], b[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const float4* q = reinterpret_cast<const float4*>(p + (size_t)s * stride);
+    a[s] = q[0];
+    b[s] = q[1];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = 0.f;
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    o[0] += a[s].x; o[1] += a[s].y; o[2] += a[s].z; o[3] += a[s].w;
+    o[4] += b[s].x; o[5] += b[s].y; o[6] += b[s].z; o[7] += b[s].w;
+  }
+}
+template <int NS>
+__device__ __forceinline__ float sum_planes1(const float* p, size_t stride) {
+  float v[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) v[s] = p[(size_t)s * stride];
+  float t = 0.f;
+#pragma unroll
+  for (int s = 0; s < NS; ++s) t += v[s];
+  return t;
+}
+__device__ __forceinline__ float sum_planes1_dyn(const float* p, size_t stride, int ns) {
+  switch (ns) {
+    case 1: return sum_planes1<1>(p, stride);
+    case 2: return sum_planes1<2>(p, stride);
+    case 4: return sum_planes1<4>(p, stride);
+    case 8: return sum_planes1<8>(p, stride);
+    case 16: return sum_planes1<16>(p, stride);
+    case 32: return sum_planes1<32>(p, stride);
+    default: {
+      // any other count: batches of 8 loads with clamped (in-bounds) plane indices
+      float t = 0.f;
+      for (int s0 = 0; s0 < ns; s0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = p[(size_t)(s0 + i < ns ? s0 + i : ns - 1) * stride];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) t += (s0 + i < ns) ? v[i] : 0.f;
+      }
+      return t;
+    }
+  }
+}
+
 // t_s[rr] = bf16(sum_s t_part[s][m][col0 + rr]) for rr < n, by the first n threads.
 __device__ __forceinline__ void stage_t(float* t_s, const LoraIn& l, int m, int M, int col0, int n) {
-  if ((int)threadIdx.x < n) {
-    float t = 0.f;
-    for (int s = 0; s < l.nsplit; ++s) t += l.t_part[((size_t)s * M + m) * l.ldt + col0 + threadIdx.x];
-    t_s[threadIdx.x] = rbf(t);
-  }
+  if ((int)threadIdx.x < n)
+    t_s[threadIdx.x] = rbf(sum_planes1_dyn(l.t_part + (size_t)m * l.ldt + col0 + threadIdx.x,
+                                           (size_t)M * l.ldt, l.nsplit));
 }
 
 // 8 adjacent outputs n0..n0+7 of one row: base = bf16(sum of the split planes) or the bf16 tensor.
@@ -44,13 +95,24 @@ __device__ __forceinline__ void load_base8(const uint16_t* y_bf16, const float* 
     unpack8(*reinterpret_cast<const uint4*>(y_bf16 + (size_t)m * N + n0), o);
     return;
   }
+  const float* p = y_part + (size_t)m * N + n0;
+  const size_t stride = (size_t)M * N;
+  switch (nsplit) {
+    case 1: sum_planes8<1>(p, stride, o); break;
+    case 2: sum_planes8<2>(p, stride, o); break;
+    case 4: sum_planes8<4>(p, stride, o); break;
+    case 8: sum_planes8<8>(p, stride, o); break;
+    case 16: sum_planes8<16>(p, stride, o); break;
+    default: {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float4* p = reinterpret_cast<const float4*>(y_part + ((size_t)s * M + m) * N + n0);
-    const float4 a = p[0], b = p[1];
-    o[0] += a.x; o[1] += a.y; o[2] += a.z; o[3] += a.w;
-    o[4] += b.x; o[5] += b.y; o[6] += b.z; o[7] += b.w;
+      for (int e = 0; e < 8; ++e) o[e] = 0.f;
+      for (int s = 0; s < nsplit; ++s) {
+        float t[8];
+        sum_planes8<1>(p + (size_t)s * stride, stride, t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] += t[e];
+      }
+    }
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = rbf(o[e]);
@@ -60,6 +122,7 @@ __device__ __forceinline__ void load_base8(const uint16_t* y_bf16, const float* 
 __device__ __forceinline__ void add_lora8(float* o, const float* t_s, const uint16_t* b, int ldb, int n0,
                                           int r, float ls) {
   float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
   for (int rr = 0; rr < r; ++rr) {
     float w[8];
     unpack8(*reinterpret_cast<const uint4*>(b + (size_t)rr * ldb + n0), w);
@@ -73,8 +136,8 @@ __device__ __forceinline__ void add_lora8(float* o, const float* t_s, const uint
 
 // One workgroup per row: h = bf16(bf16(y + delta) + residual); xn = RMSNorm(h).
 // In embedding mode it also fills this step's RoPE sin/cos table row.
-template <int CPT>  // 8-element chunks per thread, D <= 2048 * CPT
-__global__ __launch_bounds__(256) void row_norm_kernel(RowNormArgs a) {
+template <int CPT>  // 8-element chunks per thread, D <= 4096 * CPT
+__global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
   __shared__ float smem[8];
   __shared__ float t_s[TMX_MAX_RPAD];
   const int m = blockIdx.x, M = gridDim.x;
@@ -99,7 +162,7 @@ __global__ __launch_bounds__(256) void row_norm_kernel(RowNormArgs a) {
   const int nchunks = a.D >> 3;
 #pragma unroll
   for (int i = 0; i < CPT; ++i) {
-    const int c = threadIdx.x + 256 * i;
+    const int c = threadIdx.x + 512 * i;
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
     if (c < nchunks) {
@@ -122,11 +185,11 @@ __global__ __launch_bounds__(256) void row_norm_kernel(RowNormArgs a) {
     }
   }
   if (!a.norm_w) return;
-  ss = block_sum<4>(ss, smem);
+  ss = block_sum<8>(ss, smem);
   const float rms = sqrtf(ss / (float)a.D + a.eps);
 #pragma unroll
   for (int i = 0; i < CPT; ++i) {
-    const int c = threadIdx.x + 256 * i;
+    const int c = threadIdx.x + 512 * i;
     if (c < nchunks) {
       const int n0 = c * 8;
       float w[8], o[8];
@@ -142,14 +205,13 @@ __global__ __launch_bounds__(256) void row_norm_kernel(RowNormArgs a) {
 }
 
 int row_norm(hipStream_t st, const RowNormArgs& a, int M) {
-  if (a.D <= 0 || a.D % 8 || a.D > 2048 * 8) return TMX_ERR_SHAPE;
+  if (a.D <= 0 || a.D % 8 || a.D > 4096 * 4) return TMX_ERR_SHAPE;
   if (a.lora.t_part && a.lora.r > TMX_MAX_RPAD) return TMX_ERR_SHAPE;
   if (a.rope_tab && a.half > 256) return TMX_ERR_SHAPE;
-  const int cpt = (a.D / 8 + 255) / 256;
-  if (cpt <= 1) hipLaunchKernelGGL(row_norm_kernel<1>, dim3(M), dim3(256), 0, st, a);
-  else if (cpt <= 2) hipLaunchKernelGGL(row_norm_kernel<2>, dim3(M), dim3(256), 0, st, a);
-  else if (cpt <= 4) hipLaunchKernelGGL(row_norm_kernel<4>, dim3(M), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(row_norm_kernel<8>, dim3(M), dim3(256), 0, st, a);
+  const int cpt = (a.D / 8 + 511) / 512;
+  if (cpt <= 1) hipLaunchKernelGGL(row_norm_kernel<1>, dim3(M), dim3(512), 0, st, a);
+  else if (cpt <= 2) hipLaunchKernelGGL(row_norm_kernel<2>, dim3(M), dim3(512), 0, st, a);
+  else hipLaunchKernelGGL(row_norm_kernel<4>, dim3(M), dim3(512), 0, st, a);
   return check_launch();
 }
 
@@ -175,15 +237,12 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
       x1 = bf2f(a.qkv_bf16[(size_t)b * ntot + c1]);
       x2 = bf2f(a.qkv_bf16[(size_t)b * ntot + c2]);
     } else {
-      for (int s = 0; s < a.nsplit; ++s) {
-        x1 += a.qkv_part[((size_t)s * B + b) * ntot + c1];
-        x2 += a.qkv_part[((size_t)s * B + b) * ntot + c2];
-      }
-      x1 = rbf(x1);
-      x2 = rbf(x2);
+      x1 = rbf(sum_planes1_dyn(a.qkv_part + (size_t)b * ntot + c1, (size_t)B * ntot, a.nsplit));
+      x2 = rbf(sum_planes1_dyn(a.qkv_part + (size_t)b * ntot + c2, (size_t)B * ntot, a.nsplit));
     }
     if (a.lora.t_part) {
       float d1 = 0.f, d2 = 0.f;
+#pragma unroll 8
       for (int rr = 0; rr < a.lora.r; ++rr) {
         d1 = fmaf(t_s[rr], bf2f(a.lora.b[(size_t)rr * ntot + c1]), d1);
         d2 = fmaf(t_s[rr], bf2f(a.lora.b[(size_t)rr * ntot + c2]), d2);
@@ -292,6 +351,7 @@ int advance_step(hipStream_t st, int32_t* step) {
 using namespace tmx;
 
 static LoraIn make_lora(const void* t_part, int ldt, int nsplit, const void* b, int r, float ls) {
+  // nsplit: number of t planes
   LoraIn l = {};
   l.t_part = (const float*)t_part;
   l.ldt = ldt;
@@ -317,17 +377,18 @@ extern "C" int tmx_rmsnorm(void* stream, const void* x, const void* w, void* y, 
 }
 
 extern "C" int tmx_lora_residual_rmsnorm(void* stream, const void* y_bf16, const float* y_part,
-                                         int nsplit, const float* t_part, int ldt, const void* lora_b,
+                                         int nsplit, const float* t_part, int t_nsplit, int ldt,
+                                         const void* lora_b,
                                          int r, float lora_scale, const void* residual, void* x_out,
                                          const void* norm_w, void* xn_out, int M, int D, float eps,
                                          int family) {
-  if ((!y_bf16 && !y_part) || (t_part && !lora_b) || (norm_w && !xn_out)) return TMX_ERR_ARG;
+  if ((!y_bf16 && !y_part) || (t_part && (!lora_b || t_nsplit < 1)) || (norm_w && !xn_out)) return TMX_ERR_ARG;
   if (M <= 0 || (!y_bf16 && nsplit < 1)) return TMX_ERR_SHAPE;
   RowNormArgs a = {};
   a.y_bf16 = (const uint16_t*)y_bf16;
   a.y_part = y_part;
   a.nsplit = nsplit;
-  a.lora = make_lora(t_part, ldt, nsplit, lora_b, r, lora_scale);
+  a.lora = make_lora(t_part, ldt, t_nsplit, lora_b, r, lora_scale);
   a.residual = (const uint16_t*)residual;
   a.x_out = (uint16_t*)x_out;
   a.norm_w = (const uint16_t*)norm_w;
@@ -339,20 +400,20 @@ extern "C" int tmx_lora_residual_rmsnorm(void* stream, const void* y_bf16, const
 }
 
 extern "C" int tmx_rope_kv_write(void* stream, const void* qkv_bf16, const float* qkv_part, int nsplit,
-                                 const float* t_part, int ldt, const void* lora_b, int r,
+                                 const float* t_part, int t_nsplit, int ldt, const void* lora_b, int r,
                                  float lora_scale, const void* q_norm_w, const void* k_norm_w,
                                  const int32_t* positions, const int32_t* step, int buf_len, void* q_out,
                                  void* kcache, void* vcache, int B, int N, int Kh, int H, int C,
                                  float theta, float eps, int family) {
   if ((!qkv_bf16 && !qkv_part) || !positions || !step || !q_out || !kcache || !vcache ||
-      (t_part && !lora_b))
+      (t_part && (!lora_b || t_nsplit < 1)))
     return TMX_ERR_ARG;
   if (B <= 0 || N <= 0 || Kh <= 0 || C <= 0 || (!qkv_bf16 && nsplit < 1)) return TMX_ERR_SHAPE;
   RopeArgs a = {};
   a.qkv_bf16 = (const uint16_t*)qkv_bf16;
   a.qkv_part = qkv_part;
   a.nsplit = nsplit;
-  a.lora = make_lora(t_part, ldt, nsplit, lora_b, r, lora_scale);
+  a.lora = make_lora(t_part, ldt, t_nsplit, lora_b, r, lora_scale);
   a.q_norm_w = (const uint16_t*)q_norm_w;
   a.k_norm_w = (const uint16_t*)k_norm_w;
   a.positions = positions;
@@ -367,15 +428,16 @@ extern "C" int tmx_rope_kv_write(void* stream, const void* qkv_bf16, const float
 }
 
 extern "C" int tmx_swiglu(void* stream, const void* gate_up_bf16, const float* gate_up_part, int nsplit,
-                          const float* t_part, int ldt, const void* lora_b, int r, float lora_scale,
+                          const float* t_part, int t_nsplit, int ldt, const void* lora_b, int r,
+                          float lora_scale,
                           void* act, int M, int F) {
-  if ((!gate_up_bf16 && !gate_up_part) || !act || (t_part && !lora_b)) return TMX_ERR_ARG;
+  if ((!gate_up_bf16 && !gate_up_part) || !act || (t_part && (!lora_b || t_nsplit < 1))) return TMX_ERR_ARG;
   if (M <= 0 || F <= 0 || (!gate_up_bf16 && nsplit < 1)) return TMX_ERR_SHAPE;
   SwigluArgs a = {};
   a.gu_bf16 = (const uint16_t*)gate_up_bf16;
   a.gu_part = gate_up_part;
   a.nsplit = nsplit;
-  a.lora = make_lora(t_part, ldt, nsplit, lora_b, r, lora_scale);
+  a.lora = make_lora(t_part, ldt, t_nsplit, lora_b, r, lora_scale);
   a.act = (uint16_t*)act;
   a.F = F;
   return swiglu((hipStream_t)stream, a, M);

@@ -55,17 +55,22 @@ constexpr int kXStride = 72;  // bf16 elements per LDS row (64 + 8 pad)
 template <int V>
 struct IC { static constexpr int value = V; };
 
-// LORA = false: NSUB int4 column tiles per wave.  LORA = true: the block computes
-// t = x . A from dense bf16 columns of A^T [Rpad, K] (one 32-column tile per wave).
+// LORA = false: NSUB int4 column tiles per wave.  LORA = true: the block computes a K-slice
+// of t = x . A from bf16 tiles of A (one 32-column tile per wave); A is stored in MFMA
+// B-fragment order, [K/64][Rpad/32][64 lanes][4 steps][8], so a wave reads 4 KiB contiguously.
 template <int MT, int NSUB, bool LORA>
 __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[MT * 32][kXStride]) {
   // xs: 2 LDS buffers, buffer b holds activation tile i with i % 2 == b
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = lane >> 5, nl = lane & 31;
   const int KT = a.K >> 6;
-  const int split = blockIdx.y;
-  const int kb0 = split * a.kt_per_split;
-  const int kb1 = (kb0 + a.kt_per_split < KT) ? kb0 + a.kt_per_split : KT;
+  // K-slice of this block: main blocks follow blockIdx.y; the LoRA blocks of a launch cut K
+  // into lora_splits finer slices of their own so that none of them is the last to finish
+  const int slice = LORA ? ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y
+                         : (int)blockIdx.y;
+  const int per = LORA ? a.kt_per_lora_split : a.kt_per_split;
+  const int kb0 = slice * per;
+  const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
   const int kpg_shift = (a.G == 64) ? 0 : __builtin_ctz(a.G >> 6), KG = a.K / a.G;
 
   // this wave's column tiles; waves past the last tile recompute the last one (their
@@ -101,10 +106,16 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[
   }
   const u32x4_t* wsrc[NSUB];
   const uint16_t* ssrc[NSUB];
+  size_t wstep;  // 16-byte words between consecutive k-tiles of one column tile
+  if (LORA) {
+    wstep = (size_t)NT * 64 * 4;
+  } else {
+    wstep = 64;
+  }
 #pragma unroll
   for (int s = 0; s < NSUB; ++s) {
     if (LORA) {
-      wsrc[s] = reinterpret_cast<const u32x4_t*>(a.a_t + (size_t)(nbs[s] * 32 + nl) * a.K + h * 8);
+      wsrc[s] = reinterpret_cast<const u32x4_t*>(a.a_t) + ((size_t)nbs[s] * 64 + lane) * 4;
       ssrc[s] = nullptr;
     } else {
       wsrc[s] = reinterpret_cast<const u32x4_t*>(a.qw) + (size_t)nbs[s] * KT * 64 + lane;
@@ -112,11 +123,13 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[
     }
   }
 
-  constexpr int P = 4;               // tiles in flight per wave (HBM latency >> one k-tile of math)
+  // weight tiles in flight per wave (HBM latency); 8 where the registers allow two waves per SIMD
+  constexpr int PW = (!LORA && NSUB == 1 && MT <= 2) ? 8 : 4;
+  constexpr int PX = 4;              // activation tiles in flight (L2 latency)
   constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
-  u32x4_t xring[P][MT];
-  u32x4_t wring[P][NSUB][WPT];
-  uint16_t sring[P][NSUB];
+  u32x4_t xring[PX][MT];
+  u32x4_t wring[PW][NSUB][WPT];
+  uint16_t sring[PW][NSUB];
   const int nk = kb1 - kb0;
   if (nk <= 0) return;
   const int klast = kb1 - 1;
@@ -126,35 +139,20 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[
   auto load_w = [&](int kb, auto pc) __attribute__((always_inline)) {
     constexpr int p = decltype(pc)::value;
     kb = kb < klast ? kb : klast;
-#ifdef TMX_DEBUG_SAME_TILE
-    kb = kb0;
-#endif
 #pragma unroll
     for (int s = 0; s < NSUB; ++s) {
       if (LORA) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) wring[p][s][t] = wsrc[s][(size_t)kb * 8 + t * 2];
+        for (int t = 0; t < 4; ++t) wring[p][s][t] = wsrc[s][(size_t)kb * wstep + t];
       } else {
-#ifdef TMX_DEBUG_NO_WLOAD
-        wring[p][s][0] = u32x4_t{(uint32_t)kb, 0x12345678u, (uint32_t)lane, 0x9abcdef0u};
-        sring[p][s] = 0x3c00;
-#else
-        wring[p][s][0] = wsrc[s][(size_t)kb * 64];
-#ifdef TMX_DEBUG_NO_SLOAD
-        sring[p][s] = 0x3c00;
-#else
+        wring[p][s][0] = wsrc[s][(size_t)kb * wstep];
         sring[p][s] = ssrc[s][(size_t)(kb >> kpg_shift) * 32];
-#endif
-#endif
       }
     }
   };
   auto load_x = [&](int kb, auto pc) __attribute__((always_inline)) {
     constexpr int p = decltype(pc)::value;
     kb = kb < klast ? kb : klast;
-#ifdef TMX_DEBUG_SAME_X
-    kb = kb0;
-#endif
 #pragma unroll
     for (int i = 0; i < MT; ++i) xring[p][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + kb * 64);
   };
@@ -164,26 +162,27 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[
     for (int i = 0; i < MT; ++i)
       *reinterpret_cast<u32x4_t*>(&xs[buf][xrow_l[i]][xcol_l[i]]) = xring[p][i];
   };
-  // one k-tile (tile kb, ring slot p, LDS buffer p & 1): read the A fragments, consume and
-  // refill the weight slot, do the math, publish activation tile kb + 1 to the other buffer
-  auto tile_step = [&](int kb, auto pc) __attribute__((always_inline)) {
-    constexpr int p = decltype(pc)::value;
-    constexpr int p1 = (p + 1) % P;
+  // one k-tile (tile kb = kb0 + i, weight slot i % PW, activation slot i % PX, LDS buffer
+  // i & 1): read the A fragments, consume and refill the weight slot, do the math, publish
+  // activation tile kb + 1 to the other buffer
+  auto tile_step = [&](int kb, auto ic) __attribute__((always_inline)) {
+    constexpr int i = decltype(ic)::value;
+    constexpr int pw = i % PW, px1 = (i + 1) % PX;
     bf16x8_t xa[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int t = 0; t < 4; ++t)
-        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(&xs[p & 1][m * 32 + nl][t * 16 + h * 8]);
+        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(&xs[i & 1][m * 32 + nl][t * 16 + h * 8]);
     u32x4_t wc[NSUB][WPT];
     float s_c[NSUB];
 #pragma unroll
     for (int s = 0; s < NSUB; ++s) {
 #pragma unroll
-      for (int t = 0; t < WPT; ++t) wc[s][t] = wring[p][s][t];
-      s_c[s] = LORA ? 0.f : bf2f(sring[p][s]);
+      for (int t = 0; t < WPT; ++t) wc[s][t] = wring[pw][s][t];
+      s_c[s] = LORA ? 0.f : bf2f(sring[pw][s]);
     }
-    load_w(kb + P, pc);
+    load_w(kb + PW, IC<pw>{});
 #pragma unroll
     for (int s = 0; s < NSUB; ++s) {
       const float m8s = -8.f * s_c[s];
@@ -192,47 +191,43 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[
       for (int t = 0; t < 4; ++t) {
         bf16x8_t b;
         if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[s][t % WPT]);
-#ifdef TMX_DEBUG_NO_DEQUANT
-        else b = __builtin_bit_cast(bf16x8_t, wc[s][0]);
-#else
         else b = dequant_word(wd[t], s_c[s], m8s);
-#endif
 #pragma unroll
         for (int m = 0; m < MT; ++m)
-#ifdef TMX_DEBUG_NO_MFMA
-          acc[s][m][t] += __builtin_bit_cast(f32x4_t, b)[0] * __builtin_bit_cast(f32x4_t, xa[m][t])[1];
-#else
           acc[s][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[s][m], 0, 0, 0);
-#endif
       }
     }
-#ifndef TMX_DEBUG_NO_STASH
-    stash_x((p + 1) & 1, IC<p1>{});
-    load_x(kb + 1 + P, IC<p1>{});
+    stash_x((i + 1) & 1, IC<px1>{});
+    load_x(kb + 1 + PX, IC<px1>{});
     __syncthreads();
-#endif
   };
 
-  // prologue: P activation tiles and P weight tiles in flight, tile 0 published
+  // prologue: PX activation tiles and PW weight tiles in flight, tile 0 published
   load_x(kb0 + 0, IC<0>{}); load_x(kb0 + 1, IC<1>{}); load_x(kb0 + 2, IC<2>{}); load_x(kb0 + 3, IC<3>{});
   load_w(kb0 + 0, IC<0>{}); load_w(kb0 + 1, IC<1>{}); load_w(kb0 + 2, IC<2>{}); load_w(kb0 + 3, IC<3>{});
+  if (PW == 8) {
+    load_w(kb0 + 4, IC<4 % PW>{}); load_w(kb0 + 5, IC<5 % PW>{});
+    load_w(kb0 + 6, IC<6 % PW>{}); load_w(kb0 + 7, IC<7 % PW>{});
+  }
   stash_x(0, IC<0>{});
-  load_x(kb0 + P, IC<0>{});
+  load_x(kb0 + PX, IC<0>{});
   __syncthreads();
-  const int ngroups = nk / P;
+  const int ngroups = nk / 8;
   for (int g = 0; g < ngroups; ++g) {
-    const int kb = kb0 + g * P;
-    tile_step(kb + 0, IC<0>{});
-    tile_step(kb + 1, IC<1>{});
-    tile_step(kb + 2, IC<2>{});
-    tile_step(kb + 3, IC<3>{});
+    const int kb = kb0 + g * 8;
+    tile_step(kb + 0, IC<0>{}); tile_step(kb + 1, IC<1>{}); tile_step(kb + 2, IC<2>{}); tile_step(kb + 3, IC<3>{});
+    tile_step(kb + 4, IC<4>{}); tile_step(kb + 5, IC<5>{}); tile_step(kb + 6, IC<6>{}); tile_step(kb + 7, IC<7>{});
   }
   {
-    const int kb = kb0 + ngroups * P;
-    const int rem = nk - ngroups * P;
+    const int kb = kb0 + ngroups * 8;
+    const int rem = nk - ngroups * 8;
     if (rem > 0) tile_step(kb + 0, IC<0>{});
     if (rem > 1) tile_step(kb + 1, IC<1>{});
     if (rem > 2) tile_step(kb + 2, IC<2>{});
+    if (rem > 3) tile_step(kb + 3, IC<3>{});
+    if (rem > 4) tile_step(kb + 4, IC<4>{});
+    if (rem > 5) tile_step(kb + 5, IC<5>{});
+    if (rem > 6) tile_step(kb + 6, IC<6>{});
   }
 
   // epilogue: every wave owns its tiles outright
@@ -246,15 +241,15 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[
       for (int r = 0; r < 16; ++r) {
         const int row = m * 32 + acc_row(r, lane);
         if (row >= a.M) continue;
-        if (LORA) a.t_part[((size_t)split * a.M + row) * a.ldt + col] = acc[s][m][r];
+        if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = acc[s][m][r];
         else if (a.y_bf16) a.y_bf16[(size_t)row * a.N + col] = f2bf(acc[s][m][r]);
-        else a.y_part[((size_t)split * a.M + row) * a.N + col] = acc[s][m][r];
+        else a.y_part[((size_t)slice * a.M + row) * a.N + col] = acc[s][m][r];
       }
   }
 }
 
 template <int MT, int NSUB>
-__global__ __launch_bounds__(256, 2) void qlinear_mfma_kernel(QLinearArgs a) {
+__global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void qlinear_mfma_kernel(QLinearArgs a) {
   __shared__ __align__(16) uint16_t xs[2][MT * 32][kXStride];
   if ((int)blockIdx.x >= a.n_main_blocks) gemm_block<MT, 1, true>(a, xs);
   else gemm_block<MT, NSUB, false>(a, xs);
@@ -264,30 +259,42 @@ template <int MT, int NSUB>
 static int launch_qlinear(hipStream_t st, QLinearArgs a) {
   const int cols_per_block = 128 * NSUB;
   a.n_main_blocks = (a.N + cols_per_block - 1) / cols_per_block;
-  const int blocks = a.n_main_blocks + (a.a_t ? 1 : 0);
+  const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
   hipLaunchKernelGGL((qlinear_mfma_kernel<MT, NSUB>), dim3(blocks, a.nsplit), dim3(256), 0, st, a);
   return check_launch();
 }
 
-// Number of K-slices for a projection: enough workgroups to cover the chip, at
-// least 4 k-tiles per slice.
+static int slice_len(int KT, int s) { return ((KT + s - 1) / s + 3) / 4 * 4; }
+static bool slices_ok(int KT, int s) { return (KT + slice_len(KT, s) - 1) / slice_len(KT, s) == s; }
+
+// Number of K-slices for a projection: the smallest power of two that gives the chip at
+// least one workgroup per CU, with whole groups of 4 k-tiles per slice and no empty slice.
 int qlinear_num_splits(int K, int N, int M) {
   const int nsub = (N >= 16384 && M <= 64) ? 2 : 1;
   const int nblocks = (N + 128 * nsub - 1) / (128 * nsub);
   const int KT = K / 64;
-  int s = (256 + nblocks - 1) / nblocks;
-  const int smax = KT / 4 > 0 ? KT / 4 : 1;
-  if (s > smax) s = smax;
-  if (s > TMX_MAX_SPLITS) s = TMX_MAX_SPLITS;
-  if (s < 1) s = 1;
-  // slices are whole groups of 4 k-tiles; drop slices that would be empty
-  const int per = ((KT + s - 1) / s + 3) / 4 * 4;
-  return (KT + per - 1) / per;
+  int best = 1;
+  for (int s = 1; s <= TMX_MAX_SPLITS; s *= 2) {
+    if (!slices_ok(KT, s)) break;
+    best = s;
+    if (nblocks * s >= 256) break;
+  }
+  return best;
+}
+
+// Number of K-slices of the LoRA projection t = x . A: as fine as whole groups of 4 k-tiles
+// allow (at most TMX_MAX_LORA_SPLITS planes), so that no LoRA block outlasts the main blocks.
+int qlinear_num_lora_splits(int K) {
+  const int KT = K / 64;
+  for (int per = 4;; per += 4) {
+    const int n = (KT + per - 1) / per;
+    if (n <= TMX_MAX_LORA_SPLITS) return n;
+  }
 }
 
 // Host-side dispatch shared by the C entry point and the decode-step launcher.
 // Output: y_bf16 [M, N] when nsplit == 1 and y_bf16 != null, else y_part
-// [nsplit][M][N] f32 planes.  t_part: [nsplit][M][ldt] f32 (LoRA projection).
+// [nsplit][M][N] f32 planes.  t_part: [qlinear_num_lora_splits()][M][ldt] f32.
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
                  int N, int G, int Rpad, int nsplit) {
@@ -295,7 +302,9 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   if (M <= 0 || M > 128 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
   if (K % 64 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
   if (a_t && (!t_part || Rpad <= 0 || Rpad % 32 || Rpad > 128 || ldt < Rpad)) return TMX_ERR_SHAPE;
-  if (nsplit < 1 || (nsplit > 1 && !y_part)) return TMX_ERR_ARG;
+  if (nsplit < 1 || nsplit > TMX_MAX_SPLITS || (nsplit > 1 && !y_part)) return TMX_ERR_ARG;
+  const int KT = K / 64;
+  if (!slices_ok(KT, nsplit)) return TMX_ERR_SHAPE;  // an empty K-slice
   QLinearArgs a;
   a.x = (const uint16_t*)x;
   a.ldx = ldx;
@@ -308,9 +317,10 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   a.ldt = ldt;
   a.M = M; a.K = K; a.N = N; a.G = G; a.Rpad = Rpad;
   a.nsplit = nsplit;
-  const int KT = K / 64;
-  a.kt_per_split = ((KT + nsplit - 1) / nsplit + 3) / 4 * 4;
-  if ((KT + a.kt_per_split - 1) / a.kt_per_split != nsplit) return TMX_ERR_SHAPE;  // empty slice
+  a.kt_per_split = slice_len(KT, nsplit);
+  const int nls = qlinear_num_lora_splits(K);
+  a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
+  a.kt_per_lora_split = slice_len(KT, nls);
   const bool wide = (N >= 16384);
   if (M <= 32) return wide ? launch_qlinear<1, 2>(st, a) : launch_qlinear<1, 1>(st, a);
   if (M <= 64) return wide ? launch_qlinear<2, 2>(st, a) : launch_qlinear<2, 1>(st, a);
@@ -348,7 +358,8 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(const uint4* qw, cons
 // (+ residual), t[m][r] = bf16(sum_s t_part[s][m][r]).  Rounding points follow the
 // reference's bf16 einsum -> scale -> add chain.
 __global__ __launch_bounds__(256) void lora_apply_kernel(uint16_t* y, const float* y_part, int nsplit,
-                                                         const float* t_part, int ldt, const uint16_t* b,
+                                                         const float* t_part, int nlsplit, int ldt,
+                                                         const uint16_t* b,
                                                          int r, float ls, const uint16_t* res, int M,
                                                          int N) {
   const int n = blockIdx.x * 256 + threadIdx.x;
@@ -361,7 +372,7 @@ __global__ __launch_bounds__(256) void lora_apply_kernel(uint16_t* y, const floa
     float d = 0.f;
     for (int rr = 0; rr < r; ++rr) {
       float t = 0.f;
-      for (int s = 0; s < nsplit; ++s) t += t_part[((size_t)s * M + m) * ldt + rr];
+      for (int s = 0; s < nlsplit; ++s) t += t_part[((size_t)s * M + m) * ldt + rr];
       d = fmaf(rbf(t), bf2f(b[(size_t)rr * N + n]), d);
     }
     v = rbf(v + rbf(rbf(d) * ls));
@@ -386,10 +397,11 @@ extern "C" int tmx_int4_dequant(void* stream, const void* qweight, const void* s
 
 extern "C" size_t tmx_qlora_linear_workspace_bytes(int M, int K, int N) {
   const size_t s = qlinear_num_splits(K, N, M);
-  return s * (size_t)M * ((size_t)N + TMX_MAX_RPAD) * sizeof(float);
+  return (s * (size_t)M * N + (size_t)TMX_MAX_LORA_SPLITS * M * TMX_MAX_RPAD) * sizeof(float);
 }
 
 extern "C" int tmx_qlora_linear_num_splits(int M, int K, int N) { return qlinear_num_splits(K, N, M); }
+extern "C" int tmx_qlora_linear_num_lora_splits(int K) { return qlinear_num_lora_splits(K); }
 
 extern "C" int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight,
                                        const void* scales, const void* lora_a_t, float* y_part,
@@ -414,7 +426,8 @@ extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight
                         TMX_MAX_RPAD, M, K, N, G, r_pad, ns);
   if (rc != TMX_OK) return rc;
   hipLaunchKernelGGL(lora_apply_kernel, dim3((N + 255) / 256, M), dim3(256), 0, st, (uint16_t*)y, y_part,
-                     ns, lora ? t_part : nullptr, TMX_MAX_RPAD, (const uint16_t*)lora_b, r, lora_scale,
+                     ns, lora ? t_part : nullptr, qlinear_num_lora_splits(K), TMX_MAX_RPAD,
+                     (const uint16_t*)lora_b, r, lora_scale,
                      (const uint16_t*)residual, M, N);
   return check_launch();
 }

@@ -9,13 +9,14 @@ struct QLinearArgs {
   int ldx;
   const uint4* qw;         // packed int4 tiles
   const uint16_t* scales;  // [N/32][K/G][32] bf16
-  const uint16_t* a_t;     // LoRA A transposed [Rpad, K] bf16 (may be null)
+  const uint16_t* a_t;     // LoRA A in fragment order [K/64][Rpad/32][64][4][8] bf16 (may be null)
   uint16_t* y_bf16;        // [M, N] bf16 (only when nsplit == 1), else null
   float* y_part;           // [nsplit][M][N] f32 planes
-  float* t_part;           // [nsplit][M][ldt] f32 LoRA projection planes
+  float* t_part;           // [lora splits][M][ldt] f32 LoRA projection planes
   int ldt;
   int M, K, N, G, Rpad;
   int n_main_blocks, nsplit, kt_per_split;
+  int lora_blocks_per_split, kt_per_lora_split;  // finer K-slices of the LoRA projection
 };
 
 // The LoRA-B half applied by the consumer of a projection.
@@ -124,6 +125,7 @@ size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
 int head_sample(hipStream_t st, HeadArgs a);
 size_t head_partial_bytes(int M, int V);
 int qlinear_num_splits(int K, int N, int M);
+int qlinear_num_lora_splits(int K);
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
                  int N, int G, int Rpad, int nsplit);

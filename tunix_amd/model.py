@@ -253,7 +253,7 @@ class QLoRAModel:
           continue
         col = 0
         for j, (n, width) in enumerate(zip(names, pl.seg_cols)):
-          a = pl.lora_a_t[j * pl.rank:(j + 1) * pl.rank].t().contiguous()
+          a = pl.lora_a_dense()[:, j * pl.rank:(j + 1) * pl.rank].contiguous()
           b = pl.lora_b[:, col:col + width].contiguous()
           out[f'layers.{i}.{pre}.{n}.{wk}_lora_a'] = a
           out[f'layers.{i}.{pre}.{n}.{wk}_lora_b'] = b

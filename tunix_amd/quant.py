@@ -51,13 +51,16 @@ def pad32(r):
 
 
 def pack_lora_a(a_list, k):
-  """[A_i [K, r]] -> bf16 [r_pad, K]: the A matrices side by side, transposed,
-  zero-padded to a multiple of 32 rows."""
+  """[A_i [K, r]] -> bf16 [K // 64, r_pad // 32, 64, 4, 8]: the A matrices side by side,
+  zero-padded to a multiple of 32 columns, in MFMA B-fragment order: element
+  A[64 kb + 16 t + 8 h + j][32 ct + c] at [kb][ct][32 h + c][t][j]."""
   a = torch.cat([x.to(torch.bfloat16) for x in a_list], dim=1)  # [K, R]
   r = a.shape[1]
-  out = torch.zeros(pad32(r), k, dtype=torch.bfloat16, device=a.device)
-  out[:r] = a.t()
-  return out.contiguous()
+  rp = pad32(r)
+  full = torch.zeros(k, rp, dtype=torch.bfloat16, device=a.device)
+  full[:, :r] = a
+  t = full.reshape(k // 64, 4, 2, 8, rp // 32, 32)  # [kb, t, h, j, ct, c]
+  return t.permute(0, 4, 2, 5, 1, 3).reshape(k // 64, rp // 32, 64, 4, 8).contiguous()
 
 
 class PackedLinear:
@@ -78,7 +81,13 @@ class PackedLinear:
 
   @property
   def r_pad(self):
-    return 0 if self.lora_a_t is None else self.lora_a_t.shape[0]
+    return 0 if self.lora_a_t is None else self.lora_a_t.shape[1] * 32
+
+  def lora_a_dense(self):
+    """[K, r_pad] view of the packed A (inverse of pack_lora_a)."""
+    kt, ct = self.lora_a_t.shape[0], self.lora_a_t.shape[1]
+    t = self.lora_a_t.reshape(kt, ct, 2, 32, 4, 8).permute(0, 4, 2, 5, 1, 3)  # [kb, t, h, j, ct, c]
+    return t.reshape(kt * 64, ct * 32)
 
   @classmethod
   def from_dense(cls, ws, group, device, loras=None, lora_scale=0.0, bound=7.5):
