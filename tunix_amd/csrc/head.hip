@@ -70,15 +70,26 @@ __device__ __forceinline__ void lse_merge(float& mx, float& se, float mx2, float
 
 constexpr float kNegBig = -3.0e38f;
 
+template <int V>
+struct HIC { static constexpr int value = V; };
+constexpr int kHXStride = 72;  // bf16 elements per LDS row of the activation tile (64 + 8 pad)
+
+// Workgroup = 4 waves x 32 vocabulary rows.  The hidden-state k-tile x[0:M, 64 kb : 64 kb + 64]
+// is fetched once per workgroup, double-buffered in LDS and shared by the waves (MFMA B
+// fragments); head rows stream HBM -> registers through a ring of 4 k-tiles per wave.  Lane
+// (row, h) reads the 64 contiguous bytes k = 32 h .. 32 h + 31 of its row, so a k-tile of a row
+// is one 128-byte line split between two lanes; MFMA step t pairs them with x[.., 32 h + 8 t ..].
 template <int MT>
-__global__ __launch_bounds__(256) void head_kernel(HeadArgs a) {
+__global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) {
+  __shared__ __align__(16) uint16_t xs[2][MT * 32][kHXStride];
   __shared__ float s_f[4][MT * 32][4];
   __shared__ int s_i[4][MT * 32];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = lane >> 5, nl = lane & 31;
   const int tile = blockIdx.x * 4 + wave;
   const bool live = tile * 32 < a.V;
-  const int v0 = live ? tile * 32 : 0;
+  const int v0 = live ? tile * 32 : a.V - 32;  // dead waves recompute the last tile (dropped)
+  const int KT = a.D >> 6;
 
   f32x16_t acc[MT];
 #pragma unroll
@@ -86,27 +97,78 @@ __global__ __launch_bounds__(256) void head_kernel(HeadArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
 
-  const uint16_t* wrow = a.w + (size_t)(v0 + nl) * a.D + h * 32;
-  const uint16_t* xrow[MT];
+  const u32x4_t* wsrc = reinterpret_cast<const u32x4_t*>(a.w + (size_t)(v0 + nl) * a.D + h * 32);
+  const uint16_t* xsrc[MT];
+  int xrow_l[MT], xcol_l[MT];
 #pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    int row = m * 32 + nl;
-    row = row < a.M ? row : a.M - 1;
-    xrow[m] = a.x + (size_t)row * a.D + h * 32;
+  for (int i = 0; i < MT; ++i) {
+    const int c = tid + 256 * i;
+    xrow_l[i] = c >> 3;
+    xcol_l[i] = (c & 7) * 8;
+    const int row = xrow_l[i] < a.M ? xrow_l[i] : a.M - 1;
+    xsrc[i] = a.x + (size_t)row * a.D + xcol_l[i];
   }
-  if (live) {
-    for (int kb = 0; kb < a.D; kb += 64) {
-      bf16x8_t wf[4];
+  constexpr int P = 4;
+  u32x4_t wring[P][4];
+  u32x4_t xring[P][MT];
+  const int klast = KT - 1;
+  auto load_w = [&](int kb, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+    kb = kb < klast ? kb : klast;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) wf[t] = *reinterpret_cast<const bf16x8_t*>(wrow + kb + t * 8);
+    for (int t = 0; t < 4; ++t) wring[p][t] = wsrc[(size_t)kb * 8 + t];
+  };
+  auto load_x = [&](int kb, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+    kb = kb < klast ? kb : klast;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xring[p][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + kb * 64);
+  };
+  auto stash_x = [&](int buf, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      *reinterpret_cast<u32x4_t*>(&xs[buf][xrow_l[i]][xcol_l[i]]) = xring[p][i];
+  };
+  auto tile_step = [&](int kb, auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+    constexpr int p1 = (p + 1) % P;
+    bf16x8_t xf[MT][4];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        xf[m][t] = *reinterpret_cast<const bf16x8_t*>(&xs[p & 1][m * 32 + nl][h * 32 + t * 8]);
+    u32x4_t wc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) wc[t] = wring[p][t];
+    load_w(kb + P, pc);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const bf16x8_t xf = *reinterpret_cast<const bf16x8_t*>(xrow[m] + kb + t * 8);
-          acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[t], xf, acc[m], 0, 0, 0);
-        }
-    }
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wc[t]), xf[m][t],
+                                                         acc[m], 0, 0, 0);
+    stash_x((p + 1) & 1, HIC<p1>{});
+    load_x(kb + 1 + P, HIC<p1>{});
+    __syncthreads();
+  };
+  load_x(0, HIC<0>{}); load_x(1, HIC<1>{}); load_x(2, HIC<2>{}); load_x(3, HIC<3>{});
+  load_w(0, HIC<0>{}); load_w(1, HIC<1>{}); load_w(2, HIC<2>{}); load_w(3, HIC<3>{});
+  stash_x(0, HIC<0>{});
+  load_x(P, HIC<0>{});
+  __syncthreads();
+  const int ngroups = KT / P;
+  for (int g = 0; g < ngroups; ++g) {
+    const int kb = g * P;
+    tile_step(kb + 0, HIC<0>{}); tile_step(kb + 1, HIC<1>{});
+    tile_step(kb + 2, HIC<2>{}); tile_step(kb + 3, HIC<3>{});
+  }
+  {
+    const int kb = ngroups * P, rem = KT - ngroups * P;
+    if (rem > 0) tile_step(kb + 0, HIC<0>{});
+    if (rem > 1) tile_step(kb + 1, HIC<1>{});
+    if (rem > 2) tile_step(kb + 2, HIC<2>{});
   }
 
   // per-step key = fold_in(seed, step)

@@ -267,17 +267,19 @@ static int launch_qlinear(hipStream_t st, QLinearArgs a) {
 static int slice_len(int KT, int s) { return ((KT + s - 1) / s + 3) / 4 * 4; }
 static bool slices_ok(int KT, int s) { return (KT + slice_len(KT, s) - 1) / slice_len(KT, s) == s; }
 
-// Number of K-slices for a projection: the smallest power of two that gives the chip at
-// least one workgroup per CU, with whole groups of 4 k-tiles per slice and no empty slice.
+// Number of K-slices for a projection.  Wide projections (>= 192 column blocks) are not
+// split: they write bf16 directly.  Otherwise the smallest power of two that gives at least
+// 128 workgroups and at most 32 k-tiles per slice, in whole groups of 4 k-tiles, no empty slice.
 int qlinear_num_splits(int K, int N, int M) {
-  const int nsub = (N >= 16384 && M <= 64) ? 2 : 1;
-  const int nblocks = (N + 128 * nsub - 1) / (128 * nsub);
+  (void)M;
+  const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
+  if (nblocks >= 192) return 1;
   int best = 1;
   for (int s = 1; s <= TMX_MAX_SPLITS; s *= 2) {
     if (!slices_ok(KT, s)) break;
     best = s;
-    if (nblocks * s >= 256) break;
+    if (nblocks * s >= 128 && slice_len(KT, s) <= 32) break;
   }
   return best;
 }
@@ -321,7 +323,7 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   const int nls = qlinear_num_lora_splits(K);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
   a.kt_per_lora_split = slice_len(KT, nls);
-  const bool wide = (N >= 16384);
+  const bool wide = false;  // two column tiles per wave did not pay off: see the design notes
   if (M <= 32) return wide ? launch_qlinear<1, 2>(st, a) : launch_qlinear<1, 1>(st, a);
   if (M <= 64) return wide ? launch_qlinear<2, 2>(st, a) : launch_qlinear<2, 1>(st, a);
   return launch_qlinear<4, 1>(st, a);
