@@ -27,7 +27,7 @@ WORKLOADS = {
 }
 
 CLASS_NAMES = ['row_norm', 'qkv_linear', 'rope_kvwrite', 'attention', 'o_linear', 'gate_up_linear',
-               'swiglu', 'down_linear', 'head_sample', 'advance_step']
+               'swiglu', 'down_linear', 'head_sample', 'advance_step', 'empty_launch']
 
 
 def linear_bytes(pl, batch):
@@ -104,6 +104,11 @@ def main():
   ap.add_argument('--workload', default='llama3.1-8b-grpo', choices=sorted(WORKLOADS))
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--no-profile', action='store_true')
+  ap.add_argument('--sync-steps', action='store_true',
+                  help='synchronise after every decode step (counter-collection runs: the profiler '
+                       'cannot hold tens of thousands of pending dispatches)')
+  ap.add_argument('--pmc-calibrate', action='store_true',
+                  help='also run one 1 GiB device copy (a kernel of known traffic) to scale PMC counters')
   args = ap.parse_args()
   if args.gpus != 1:
     print('bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1',
@@ -143,14 +148,27 @@ def main():
   def fresh_state():
     st = sampler.init_sample_state(ids, prompt + new, False, None, temp, top_p, None, 0,
                                    include_logprobs=True, prompt_lengths=np.full(batch, prompt))
-    sampler.run_steps(st, prompt - 1, sample=False)  # cache fill over the prompt (untimed)
+    run(st, prompt - 1, False)  # cache fill over the prompt (untimed)
     return st
 
+  def run(st, n, sample=True):
+    if not args.sync_steps:
+      return sampler.run_steps(st, n, sample=sample)
+    for _ in range(n):
+      sampler.run_steps(st, 1, sample=sample)
+      torch.cuda.synchronize()
+
+  if args.pmc_calibrate:
+    src = torch.empty(1 << 30, dtype=torch.uint8, device='cuda')
+    dst = torch.empty_like(src)
+    dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+    torch.cuda.synchronize()
+    del src, dst
   st = fresh_state()
-  sampler.run_steps(st, args.warmup, sample=True)
+  run(st, args.warmup)
   torch.cuda.synchronize()
   t0 = time.perf_counter()
-  sampler.run_steps(st, args.steps, sample=True)
+  run(st, args.steps)
   torch.cuda.synchronize()
   dt = time.perf_counter() - t0
   toks = st['token_buffer'][:, prompt:prompt + args.warmup + args.steps]
@@ -217,8 +235,6 @@ def main():
       done_steps += 1
     per_step = tot_ms / max(ctx_n, 1)
     result['kernel_ms_per_step'] = {n: round(float(v), 4) for n, v in zip(CLASS_NAMES, per_step)}
-    dom = int(np.argmax(tot_ms))
-    avg_ms = float(tot_ms[dom] / max(tot_cnt[dom], 1))
     layer0 = model.layers[0]
     ctx = ctx_sum / max(ctx_n, 1)
     alg = {
@@ -228,16 +244,53 @@ def main():
         'attention': batch * ctx * cfg.num_kv_heads * cfg.head_dim * 2 * 2,
         'head_sample': hbytes,
     }
-    if CLASS_NAMES[dom] in alg:
-      a = alg[CLASS_NAMES[dom]] / (avg_ms * 1e-3) / 1e9
-      result['roofline'] = {'bound': 'hbm', 'achieved': a, 'peak': 8000.0, 'unit': 'GB/s',
-                            'frac': a / 8000.0, 'traffic': None, 'kernel': CLASS_NAMES[dom],
-                            'avg_launch_ms': avg_ms, 'algorithmic_bytes_per_launch': alg[CLASS_NAMES[dom]]}
-    result['roofline_all'] = {
-        n: {'avg_launch_ms': float(tot_ms[i] / max(tot_cnt[i], 1)),
-            'achieved_GBps': alg[n] / (float(tot_ms[i] / max(tot_cnt[i], 1)) * 1e-3) / 1e9,
-            'frac': alg[n] / (float(tot_ms[i] / max(tot_cnt[i], 1)) * 1e-3) / 8e12}
-        for i, n in enumerate(CLASS_NAMES) if n in alg and tot_cnt[i] > 0}
+    # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
+    mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
+    symbols = {
+        f'tmx::qlinear_mfma_kernel<{mt}>': ['qkv_linear', 'o_linear', 'gate_up_linear', 'down_linear'],
+        f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention'],
+        f'tmx::head_kernel<{mt}>': ['head_sample'],
+    }
+    idx = {n: i for i, n in enumerate(CLASS_NAMES)}
+    # An event pair around a launch also times the packet processing on both sides of it, so it
+    # reads a few microseconds above rocprofv3's kernel trace (which brackets the dispatch
+    # alone).  The pair around a kernel that does nothing is reported beside it as the upper
+    # bound of that excess; the roofline figures use the uncorrected (longer) event time.
+    pair_ms = float(tot_ms[idx['empty_launch']] / max(tot_cnt[idx['empty_launch']], 1))
+    per_symbol = {}
+    for sym, classes in symbols.items():
+      t = float(sum(tot_ms[idx[c]] for c in classes))
+      n = int(sum(tot_cnt[idx[c]] for c in classes))
+      if n == 0:
+        continue
+      launches_per_class = {c: int(tot_cnt[idx[c]]) for c in classes}
+      byts = float(sum(alg[c] * launches_per_class[c] for c in classes)) / n
+      avg = t / n
+      per_symbol[sym] = {'total_ms_per_step': avg * n / max(ctx_n, 1), 'launches_per_step': n / max(ctx_n, 1),
+                         'avg_launch_ms': avg,
+                         'algorithmic_bytes_per_launch': byts,
+                         'achieved_GBps': byts / (avg * 1e-3) / 1e9, 'frac': byts / (avg * 1e-3) / 8e12}
+    dom = max(per_symbol, key=lambda k: per_symbol[k]['total_ms_per_step'])
+    traffic = None
+    tpath = os.path.join(ROOT, 'profiles', 'traffic.json')
+    if os.path.exists(tpath):  # HBM bytes per launch from the rocprofv3 --pmc runs (see profiles/)
+      traffic = json.load(open(tpath)).get(args.workload, {}).get(dom)
+    d = per_symbol[dom]
+    result['roofline'] = {'bound': 'hbm', 'achieved': d['achieved_GBps'], 'peak': 8000.0, 'unit': 'GB/s',
+                          'frac': d['frac'], 'traffic': traffic, 'kernel': dom,
+                          'avg_launch_ms': d['avg_launch_ms'],
+                          'empty_launch_event_pair_ms': pair_ms,
+                          'algorithmic_bytes_per_launch': d['algorithmic_bytes_per_launch'],
+                          'note': 'mean HIP-event time around the launches of this kernel in the sampled '
+                                  'steps (includes event packet processing, see empty_launch_event_pair_ms); '
+                                  'the projection kernel serves qkv, o, gate|up and down'}
+    result['roofline_kernels'] = per_symbol
+    result['roofline_all'] = {}
+    for i, n in enumerate(CLASS_NAMES):
+      if n in alg and tot_cnt[i] > 0:
+        avg = float(tot_ms[i] / tot_cnt[i])
+        result['roofline_all'][n] = {'avg_launch_ms': avg, 'achieved_GBps': alg[n] / (avg * 1e-3) / 1e9,
+                                     'frac': alg[n] / (avg * 1e-3) / 8e12}
 
   if not args.no_cpu_baseline:
     del st

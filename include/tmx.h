@@ -221,7 +221,9 @@ int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state,
 /* Measurement aid (no counterpart in the reference): the same as tmx_decode_steps, but every
  * kernel launch is bracketed by HIP events on `stream`; after enqueuing, the call SYNCHRONISES
  * the stream and adds up the elapsed milliseconds and the launch count per kernel class into
- * the two HOST arrays of TMX_NUM_KERNEL_CLASSES entries. */
+ * the two HOST arrays of TMX_NUM_KERNEL_CLASSES entries.  An event pair around a launch also
+ * times the packet processing before and after it; class TMX_K_EMPTY brackets a kernel that
+ * does nothing (once per layer), so that callers can subtract that constant. */
 #define TMX_K_ROWNORM 0  /* embedding gather / residual + LoRA-B + RMSNorm rows */
 #define TMX_K_QKV 1      /* fused q|k|v int4 projection (+ LoRA-A tiles) */
 #define TMX_K_ROPE 2     /* LoRA-B + RoPE + KV-cache write */
@@ -232,7 +234,8 @@ int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state,
 #define TMX_K_DOWN 7     /* down projection */
 #define TMX_K_HEAD 8     /* head + log-softmax + token selection (+ finalize) */
 #define TMX_K_ADVANCE 9
-#define TMX_NUM_KERNEL_CLASSES 10
+#define TMX_K_EMPTY 10   /* one empty launch per layer: what an event pair costs by itself */
+#define TMX_NUM_KERNEL_CLASSES 11
 int tmx_decode_steps_profiled(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
                               int n_steps, int sample, float* class_ms_host, int* class_launches_host);
 

@@ -227,6 +227,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
         TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
       }
+      if (prof) TMX_TRY(TMX_K_EMPTY, empty_launch(st));
     }
     if (sample) {
       HeadArgs a = {};

@@ -41,226 +41,186 @@ __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s)
 }
 
 
-// One workgroup = 4 waves owns a block of 4 * NSUB adjacent 32-column tiles (one
-// group of NSUB tiles per wave) over one K-slice.  The activation k-tile
-// x[0:M, 64 kb : 64 kb + 64] is fetched once per workgroup with coalesced 16-byte
-// loads, double-buffered in LDS (rows padded to 144 bytes: conflict-free
-// ds_read_b128) and shared by the four waves as MFMA A fragments; weights go
-// HBM -> registers.  Global loads of k-tile i+1 are issued before the MFMAs of
-// k-tile i.  Small-N projections are split along K over blockIdx.y so that
-// every CU streams weights; each split writes its own f32 plane (summed by the
-// consumer kernel), so results do not depend on scheduling order.
-constexpr int kXStride = 72;  // bf16 elements per LDS row (64 + 8 pad)
+// One workgroup = 4 waves owns a block of 4 adjacent 32-column tiles (one per wave) over one
+// K-slice and advances in steps of KS = 4 k-tiles (256 k).  Per step the activation slab
+// x[0:M, 256 s : 256 s + 256] is fetched once per workgroup with coalesced 16-byte loads
+// (issued one step ahead), double-buffered in LDS (rows padded by 16 bytes: conflict-free
+// ds_read_b128) and shared by the four waves as MFMA A fragments; weights go HBM -> registers
+// through a ring that keeps two steps (8 tiles, 8 KiB per wave) in flight.  One barrier per
+// step amortises the synchronisation over four tiles.  Small-N projections are split along
+// K over blockIdx.y so that every CU streams weights; each split writes its own f32 plane
+// (summed by the consumer kernel), so results do not depend on scheduling order.
+constexpr int kKS = 4;                    // k-tiles per pipeline step
+constexpr int kXStride = kKS * 64 + 8;    // bf16 elements per LDS row
 
 template <int V>
 struct IC { static constexpr int value = V; };
 
-// LORA = false: NSUB int4 column tiles per wave.  LORA = true: the block computes a K-slice
+// LORA = false: one int4 column tile per wave.  LORA = true: the block computes a K-slice
 // of t = x . A from bf16 tiles of A (one 32-column tile per wave); A is stored in MFMA
 // B-fragment order, [K/64][Rpad/32][64 lanes][4 steps][8], so a wave reads 4 KiB contiguously.
-template <int MT, int NSUB, bool LORA>
+template <int MT, bool LORA>
 __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[MT * 32][kXStride]) {
-  // xs: 2 LDS buffers, buffer b holds activation tile i with i % 2 == b
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = lane >> 5, nl = lane & 31;
   const int KT = a.K >> 6;
   // K-slice of this block: main blocks follow blockIdx.y; the LoRA blocks of a launch cut K
-  // into lora_splits finer slices of their own so that none of them is the last to finish
+  // into finer slices of their own so that none of them is the last to finish
   const int slice = LORA ? ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y
                          : (int)blockIdx.y;
   const int per = LORA ? a.kt_per_lora_split : a.kt_per_split;
   const int kb0 = slice * per;
   const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
+  const int nsteps = (kb1 - kb0) / kKS;  // slices are whole steps (host guarantees K % 256 == 0)
+  if (nsteps <= 0) return;
   const int kpg_shift = (a.G == 64) ? 0 : __builtin_ctz(a.G >> 6), KG = a.K / a.G;
 
-  // this wave's column tiles; waves past the last tile recompute the last one (their
-  // results are dropped) so that the pipelined loop below stays free of branches
+  // this wave's column tile; waves past the last tile recompute the last one (result dropped)
   const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
-  const int nb_first = LORA ? wave : ((int)blockIdx.x * 4 + wave) * NSUB;
-  int nbs[NSUB];
-  bool sub_ok[NSUB];
-#pragma unroll
-  for (int s = 0; s < NSUB; ++s) {
-    sub_ok[s] = (nb_first + s) < NT;
-    nbs[s] = sub_ok[s] ? nb_first + s : NT - 1;
-  }
+  const int nb_mine = LORA ? wave : (int)blockIdx.x * 4 + wave;
+  const bool tile_ok = nb_mine < NT;
+  const int nb = tile_ok ? nb_mine : NT - 1;
 
-  f32x16_t acc[NSUB][MT];
+  f32x16_t acc[MT];
 #pragma unroll
-  for (int s = 0; s < NSUB; ++s)
+  for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[s][m][r] = 0.f;
+    for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
 
-  // cooperative activation load: chunk c = tid + 256 i -> row c / 8, 16-byte column c % 8
-  const uint16_t* xsrc[MT];
-  int xrow_l[MT], xcol_l[MT];
+  // cooperative activation load: chunk c = tid + 256 i -> row c / 32, 16-byte column c % 32
+  constexpr int XC = MT * 4;  // chunks per thread and step
+  const uint16_t* xsrc[XC];
+  int xoff_l[XC];
 #pragma unroll
-  for (int i = 0; i < MT; ++i) {
+  for (int i = 0; i < XC; ++i) {
     const int c = tid + 256 * i;
-    xrow_l[i] = c >> 3;
-    xcol_l[i] = (c & 7) * 8;
-    const int row = xrow_l[i] < a.M ? xrow_l[i] : a.M - 1;
-    xsrc[i] = a.x + (size_t)row * a.ldx + xcol_l[i];
+    const int row_l = c >> 5, col_l = (c & 31) * 8;
+    xoff_l[i] = row_l * kXStride + col_l;
+    const int row = row_l < a.M ? row_l : a.M - 1;
+    xsrc[i] = a.x + (size_t)row * a.ldx + (size_t)kb0 * 64 + col_l;
   }
-  const u32x4_t* wsrc[NSUB];
-  const uint16_t* ssrc[NSUB];
+  constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
+  constexpr int DW = LORA ? 1 : 2;   // steps of weights in flight
+  const u32x4_t* wsrc;
+  const uint16_t* ssrc = nullptr;
   size_t wstep;  // 16-byte words between consecutive k-tiles of one column tile
   if (LORA) {
     wstep = (size_t)NT * 64 * 4;
+    wsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + ((size_t)nb * 64 + lane) * 4 + (size_t)kb0 * wstep;
   } else {
     wstep = 64;
+    wsrc = reinterpret_cast<const u32x4_t*>(a.qw) + (size_t)nb * KT * 64 + lane + (size_t)kb0 * wstep;
+    ssrc = a.scales + (size_t)nb * KG * 32 + nl;
   }
-#pragma unroll
-  for (int s = 0; s < NSUB; ++s) {
-    if (LORA) {
-      wsrc[s] = reinterpret_cast<const u32x4_t*>(a.a_t) + ((size_t)nbs[s] * 64 + lane) * 4;
-      ssrc[s] = nullptr;
-    } else {
-      wsrc[s] = reinterpret_cast<const u32x4_t*>(a.qw) + (size_t)nbs[s] * KT * 64 + lane;
-      ssrc[s] = a.scales + (size_t)nbs[s] * KG * 32 + nl;
-    }
-  }
+  u32x4_t xreg[XC];
+  u32x4_t wring[DW][kKS][WPT];
+  uint16_t sring[DW][kKS];
+  const int last_step = nsteps - 1;
 
-  // weight tiles in flight per wave (HBM latency); 8 where the registers allow two waves per SIMD
-  constexpr int PW = (!LORA && NSUB == 1 && MT <= 2) ? 8 : 4;
-  constexpr int PX = 4;              // activation tiles in flight (L2 latency)
-  constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
-  u32x4_t xring[PX][MT];
-  u32x4_t wring[PW][NSUB][WPT];
-  uint16_t sring[PW][NSUB];
-  const int nk = kb1 - kb0;
-  if (nk <= 0) return;
-  const int klast = kb1 - 1;
-
-  // Unconditional loads with clamped tile indices: the compiler can then count the
+  // Unconditional loads with clamped step indices: the compiler can then count the
   // outstanding loads exactly and wait only for the oldest one.
-  auto load_w = [&](int kb, auto pc) __attribute__((always_inline)) {
-    constexpr int p = decltype(pc)::value;
-    kb = kb < klast ? kb : klast;
+  auto load_w_tile = [&](int step, auto dc, auto kc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, kt = decltype(kc)::value;
+    step = step < last_step ? step : last_step;
+    const int rel = step * kKS + kt;  // k-tile relative to kb0
 #pragma unroll
-    for (int s = 0; s < NSUB; ++s) {
-      if (LORA) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) wring[p][s][t] = wsrc[s][(size_t)kb * wstep + t];
-      } else {
-        wring[p][s][0] = wsrc[s][(size_t)kb * wstep];
-        sring[p][s] = ssrc[s][(size_t)(kb >> kpg_shift) * 32];
-      }
-    }
+    for (int t = 0; t < WPT; ++t) wring[d][kt][t] = wsrc[(size_t)rel * wstep + t];
+    if (!LORA) sring[d][kt] = ssrc[(size_t)((kb0 + rel) >> kpg_shift) * 32];
   };
-  auto load_x = [&](int kb, auto pc) __attribute__((always_inline)) {
-    constexpr int p = decltype(pc)::value;
-    kb = kb < klast ? kb : klast;
-#pragma unroll
-    for (int i = 0; i < MT; ++i) xring[p][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + kb * 64);
+  auto load_w = [&](int step, auto dc) __attribute__((always_inline)) {
+    load_w_tile(step, dc, IC<0>{}); load_w_tile(step, dc, IC<1>{});
+    load_w_tile(step, dc, IC<2>{}); load_w_tile(step, dc, IC<3>{});
   };
-  auto stash_x = [&](int buf, auto pc) __attribute__((always_inline)) {
-    constexpr int p = decltype(pc)::value;
+  auto load_x = [&](int step) __attribute__((always_inline)) {
+    step = step < last_step ? step : last_step;
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-      *reinterpret_cast<u32x4_t*>(&xs[buf][xrow_l[i]][xcol_l[i]]) = xring[p][i];
+    for (int i = 0; i < XC; ++i)
+      xreg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + (size_t)step * kKS * 64);
   };
-  // one k-tile (tile kb = kb0 + i, weight slot i % PW, activation slot i % PX, LDS buffer
-  // i & 1): read the A fragments, consume and refill the weight slot, do the math, publish
-  // activation tile kb + 1 to the other buffer
-  auto tile_step = [&](int kb, auto ic) __attribute__((always_inline)) {
-    constexpr int i = decltype(ic)::value;
-    constexpr int pw = i % PW, px1 = (i + 1) % PX;
+  auto stash_x = [&](int buf) __attribute__((always_inline)) {
+    uint16_t* base = &xs[buf][0][0];
+#pragma unroll
+    for (int i = 0; i < XC; ++i) *reinterpret_cast<u32x4_t*>(base + xoff_l[i]) = xreg[i];
+  };
+  // one of the four k-tiles of a step
+  auto tile_math = [&](int step, int buf, auto dc, auto kc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, kt = decltype(kc)::value;
     bf16x8_t xa[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int t = 0; t < 4; ++t)
-        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(&xs[i & 1][m * 32 + nl][t * 16 + h * 8]);
-    u32x4_t wc[NSUB][WPT];
-    float s_c[NSUB];
+        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(&xs[buf][m * 32 + nl][kt * 64 + t * 16 + h * 8]);
+    u32x4_t wc[WPT];
 #pragma unroll
-    for (int s = 0; s < NSUB; ++s) {
+    for (int t = 0; t < WPT; ++t) wc[t] = wring[d][kt][t];
+    const float s_c = LORA ? 0.f : bf2f(sring[d][kt]);
+    load_w_tile(step + DW, dc, kc);  // slot consumed: refill it DW steps ahead
+    const float m8s = -8.f * s_c;
+    const uint32_t wd[4] = {wc[0].x, wc[0].y, wc[0].z, wc[0].w};
 #pragma unroll
-      for (int t = 0; t < WPT; ++t) wc[s][t] = wring[pw][s][t];
-      s_c[s] = LORA ? 0.f : bf2f(sring[pw][s]);
+    for (int t = 0; t < 4; ++t) {
+      bf16x8_t b;
+      if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[t % WPT]);
+      else b = dequant_word(wd[t], s_c, m8s);
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[m], 0, 0, 0);
     }
-    load_w(kb + PW, IC<pw>{});
-#pragma unroll
-    for (int s = 0; s < NSUB; ++s) {
-      const float m8s = -8.f * s_c[s];
-      const uint32_t wd[4] = {wc[s][0].x, wc[s][0].y, wc[s][0].z, wc[s][0].w};
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        bf16x8_t b;
-        if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[s][t % WPT]);
-        else b = dequant_word(wd[t], s_c[s], m8s);
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-          acc[s][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[s][m], 0, 0, 0);
-      }
-    }
-    stash_x((i + 1) & 1, IC<px1>{});
-    load_x(kb + 1 + PX, IC<px1>{});
+  };
+  // step s: activations in LDS buffer s & 1, weights in ring slot s % DW
+  auto do_step = [&](int step, auto sc) __attribute__((always_inline)) {
+    constexpr int sp = decltype(sc)::value;  // step parity (static)
+    constexpr int d = sp % DW;
+    load_x(step + 1);
+    tile_math(step, sp, IC<d>{}, IC<0>{});
+    tile_math(step, sp, IC<d>{}, IC<1>{});
+    tile_math(step, sp, IC<d>{}, IC<2>{});
+    tile_math(step, sp, IC<d>{}, IC<3>{});
+    stash_x(sp ^ 1);
     __syncthreads();
   };
 
-  // prologue: PX activation tiles and PW weight tiles in flight, tile 0 published
-  load_x(kb0 + 0, IC<0>{}); load_x(kb0 + 1, IC<1>{}); load_x(kb0 + 2, IC<2>{}); load_x(kb0 + 3, IC<3>{});
-  load_w(kb0 + 0, IC<0>{}); load_w(kb0 + 1, IC<1>{}); load_w(kb0 + 2, IC<2>{}); load_w(kb0 + 3, IC<3>{});
-  if (PW == 8) {
-    load_w(kb0 + 4, IC<4 % PW>{}); load_w(kb0 + 5, IC<5 % PW>{});
-    load_w(kb0 + 6, IC<6 % PW>{}); load_w(kb0 + 7, IC<7 % PW>{});
-  }
-  stash_x(0, IC<0>{});
-  load_x(kb0 + PX, IC<0>{});
+  load_x(0);
+  load_w(0, IC<0>{});
+  if (DW == 2) load_w(1, IC<1 % DW>{});
+  stash_x(0);
   __syncthreads();
-  const int ngroups = nk / 8;
-  for (int g = 0; g < ngroups; ++g) {
-    const int kb = kb0 + g * 8;
-    tile_step(kb + 0, IC<0>{}); tile_step(kb + 1, IC<1>{}); tile_step(kb + 2, IC<2>{}); tile_step(kb + 3, IC<3>{});
-    tile_step(kb + 4, IC<4>{}); tile_step(kb + 5, IC<5>{}); tile_step(kb + 6, IC<6>{}); tile_step(kb + 7, IC<7>{});
+  const int npairs = nsteps / 2;
+  for (int g = 0; g < npairs; ++g) {
+    do_step(2 * g, IC<0>{});
+    do_step(2 * g + 1, IC<1>{});
   }
-  {
-    const int kb = kb0 + ngroups * 8;
-    const int rem = nk - ngroups * 8;
-    if (rem > 0) tile_step(kb + 0, IC<0>{});
-    if (rem > 1) tile_step(kb + 1, IC<1>{});
-    if (rem > 2) tile_step(kb + 2, IC<2>{});
-    if (rem > 3) tile_step(kb + 3, IC<3>{});
-    if (rem > 4) tile_step(kb + 4, IC<4>{});
-    if (rem > 5) tile_step(kb + 5, IC<5>{});
-    if (rem > 6) tile_step(kb + 6, IC<6>{});
-  }
+  if (nsteps & 1) do_step(nsteps - 1, IC<0>{});
 
-  // epilogue: every wave owns its tiles outright
-#pragma unroll
-  for (int s = 0; s < NSUB; ++s) {
-    if (!sub_ok[s]) continue;
-    const int col = (nb_first + s) * 32 + nl;
+  // epilogue: every wave owns its tile outright
+  if (tile_ok) {
+    const int col = nb_mine * 32 + nl;
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m * 32 + acc_row(r, lane);
         if (row >= a.M) continue;
-        if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = acc[s][m][r];
-        else if (a.y_bf16) a.y_bf16[(size_t)row * a.N + col] = f2bf(acc[s][m][r]);
-        else a.y_part[((size_t)slice * a.M + row) * a.N + col] = acc[s][m][r];
+        if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = acc[m][r];
+        else if (a.y_bf16) a.y_bf16[(size_t)row * a.N + col] = f2bf(acc[m][r]);
+        else a.y_part[((size_t)slice * a.M + row) * a.N + col] = acc[m][r];
       }
   }
 }
 
-template <int MT, int NSUB>
+template <int MT>
 __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void qlinear_mfma_kernel(QLinearArgs a) {
   __shared__ __align__(16) uint16_t xs[2][MT * 32][kXStride];
-  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block<MT, 1, true>(a, xs);
-  else gemm_block<MT, NSUB, false>(a, xs);
+  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block<MT, true>(a, xs);
+  else gemm_block<MT, false>(a, xs);
 }
 
-template <int MT, int NSUB>
+template <int MT>
 static int launch_qlinear(hipStream_t st, QLinearArgs a) {
-  const int cols_per_block = 128 * NSUB;
-  a.n_main_blocks = (a.N + cols_per_block - 1) / cols_per_block;
+  a.n_main_blocks = (a.N + 127) / 128;
   const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
-  hipLaunchKernelGGL((qlinear_mfma_kernel<MT, NSUB>), dim3(blocks, a.nsplit), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((qlinear_mfma_kernel<MT>), dim3(blocks, a.nsplit), dim3(256), 0, st, a);
   return check_launch();
 }
 
@@ -302,7 +262,7 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
                  int N, int G, int Rpad, int nsplit) {
   if (!x || !qw || !scales || (!y_bf16 && !y_part)) return TMX_ERR_ARG;
   if (M <= 0 || M > 128 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
-  if (K % 64 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
+  if (K % 256 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
   if (a_t && (!t_part || Rpad <= 0 || Rpad % 32 || Rpad > 128 || ldt < Rpad)) return TMX_ERR_SHAPE;
   if (nsplit < 1 || nsplit > TMX_MAX_SPLITS || (nsplit > 1 && !y_part)) return TMX_ERR_ARG;
   const int KT = K / 64;
@@ -323,10 +283,9 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   const int nls = qlinear_num_lora_splits(K);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
   a.kt_per_lora_split = slice_len(KT, nls);
-  const bool wide = false;  // two column tiles per wave did not pay off: see the design notes
-  if (M <= 32) return wide ? launch_qlinear<1, 2>(st, a) : launch_qlinear<1, 1>(st, a);
-  if (M <= 64) return wide ? launch_qlinear<2, 2>(st, a) : launch_qlinear<2, 1>(st, a);
-  return launch_qlinear<4, 1>(st, a);
+  if (M <= 32) return launch_qlinear<1>(st, a);
+  if (M <= 64) return launch_qlinear<2>(st, a);
+  return launch_qlinear<4>(st, a);
 }
 
 // ---------------------------------------------------------------------------

@@ -120,6 +120,7 @@ int row_norm(hipStream_t st, const RowNormArgs& a, int M);
 int rope_kvwrite(hipStream_t st, const RopeArgs& a, int B);
 int swiglu(hipStream_t st, const SwigluArgs& a, int M);
 int advance_step(hipStream_t st, int32_t* step);
+int empty_launch(hipStream_t st);  // measurement aid: a kernel that does nothing
 int gqa_decode(hipStream_t st, AttnArgs a, int H);
 size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
 int head_sample(hipStream_t st, HeadArgs a);
