@@ -1,6 +1,6 @@
 """Per-kernel means of one hardware counter from a rocprofv3 counter-collection CSV.
 
-  python -m tunix_amd.pmc_summary <..._counter_collection.csv> FETCH_SIZE [--scale S]
+  python -m tunix_amd.pmc_summary <..._counter_collection.csv> FETCH_SIZE [--scale S] [--match TEXT]
 
 prints, for every kernel symbol, the number of dispatches and the mean / max of
 the counter over them (times S, the calibration factor of a copy of known
@@ -13,11 +13,11 @@ import csv
 import json
 
 
-def summarize(path, counter, scale=1.0):
+def summarize(path, counter, scale=1.0, match=None):
   agg = collections.defaultdict(list)
   with open(path) as f:
     for row in csv.DictReader(f):
-      if row['Counter_Name'] != counter:
+      if row['Counter_Name'] != counter or (match and match not in row['Kernel_Name']):
         continue
       agg[row['Kernel_Name'].split('(')[0]].append(float(row['Counter_Value']) * scale)
   return {k: {'launches': len(v), 'mean': sum(v) / len(v), 'max': max(v)} for k, v in agg.items()}
@@ -30,8 +30,9 @@ def main():
   ap.add_argument('--scale', type=float, default=1.0)
   ap.add_argument('--json', action='store_true')
   ap.add_argument('--top', type=int, default=16)
+  ap.add_argument('--match', default=None, help='only kernels whose name contains this text')
   a = ap.parse_args()
-  s = summarize(a.csv, a.counter, a.scale)
+  s = summarize(a.csv, a.counter, a.scale, a.match)
   if a.json:
     print(json.dumps(s))
     return
