@@ -149,6 +149,22 @@ int tmx_head_sample(void* stream, const void* x, const void* head_w, int M, int 
                     int32_t* token_buffer, float* logprobs, uint8_t* done, int buf_len,
                     float* logits_out, void* workspace);
 
+/* The sorting branch of sample_top_p (top_p < 1 and / or top_k > 0),
+ * tunix/generate/sampler.py:136-153: candidates = the top_k (or all V) logits in descending
+ * order, ties in index order; probs = softmax over the candidates; a candidate is dropped when
+ * the cumulative probability before it exceeds top_p; token = Gumbel-max over the survivors
+ * with the noise of rank i of row m drawn at linear index m * k + i; logprob =
+ * log_softmax(z)[token] over the full vocabulary.  Same outputs as tmx_head_sample.
+ * nucleus_workspace: tmx_nucleus_workspace_bytes(M, V) bytes (sort keys, sorted pairs and the
+ * radix sort's scratch; the size is asked of the sort routine and is 0 without a device). */
+size_t tmx_nucleus_workspace_bytes(int M, int V);
+int tmx_head_sample_nucleus(void* stream, const void* x, const void* head_w, int M, int D, int V,
+                            float temperature, float top_p, int top_k, uint32_t seed_hi,
+                            uint32_t seed_lo, const int32_t* step, const int32_t* forbidden,
+                            int n_forbidden, const int32_t* eos, int n_eos, int32_t* token_buffer,
+                            float* logprobs, uint8_t* done, int buf_len, void* workspace,
+                            void* nucleus_workspace, size_t nucleus_workspace_bytes);
+
 /* ---- whole decode steps ------------------------------------------------------ */
 
 
@@ -206,6 +222,8 @@ typedef struct {
   float* logits_out;     /* optional f32 [B, V]: logits of the last executed step */
   void* workspace;
   size_t workspace_bytes;
+  void* nucleus_workspace; /* tmx_nucleus_workspace_bytes(B, V); needed when top_p < 1 or top_k > 0 */
+  size_t nucleus_workspace_bytes;
 } tmx_decode_state;
 
 size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int cache_size);

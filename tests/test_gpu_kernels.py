@@ -332,6 +332,112 @@ def test_head_temperature_sampling_matches_threefry_oracle(M, D, V, temp):
     assert (tok3[:, step + 1] != tok[:, step + 1]).mean() > 0.5
 
 
+def _run_nucleus(x, w, temperature, top_p, top_k, key, step, forbidden=(), eos=(-1,), col_len=20):
+  T = G.Keep()
+  M, D = x.shape
+  V = w.shape[0]
+  lib = _lib.lib()
+  ws = torch.empty(lib.tmx_head_sample_workspace_bytes(M, V), dtype=torch.uint8, device=G.DEV)
+  nb = lib.tmx_nucleus_workspace_bytes(M, V)
+  assert nb > 0
+  nws = torch.empty(nb, dtype=torch.uint8, device=G.DEV)
+  tok = torch.full((M, col_len), -5, dtype=torch.int32, device=G.DEV)
+  lp = torch.zeros(M, col_len, dtype=torch.float32, device=G.DEV)
+  done = torch.zeros(M, dtype=torch.uint8, device=G.DEV)
+  fb = T.i32(list(forbidden)) if forbidden else None
+  G.call('tmx_head_sample_nucleus', S(), T.bf(x), T.bf(w), M, D, V, temperature, top_p, top_k or 0,
+         int(key[0]), int(key[1]), T.i32([step]), fb, len(forbidden), T.i32(list(eos)), len(eos), G.p(tok),
+         G.p(lp), G.p(done), col_len, G.p(ws), G.p(nws), nb)
+  G.sync()
+  return tok.cpu().numpy(), lp.cpu().numpy(), done.cpu().numpy()
+
+
+def _nucleus_clear_rows(z, key, top_p, top_k):
+  """Rows whose outcome cannot flip on f32 rounding: the cut is not within 8e-6 of top_p (the
+  running sum is accumulated in another order on the GPU) and the winning noisy key leads by 1e-4."""
+  k = z.shape[1] if not top_k else top_k
+  order = np.argsort(-z, axis=-1, kind='stable')[:, :k]
+  zs = np.take_along_axis(z, order, axis=-1)
+  ps = OS.softmax(zs)
+  cs = np.cumsum(ps, axis=-1, dtype=np.float32)
+  gap = np.abs((cs - ps) - np.float32(top_p)).min(axis=-1)
+  keep = ~((cs - ps) > np.float32(top_p))
+  noisy = np.where(keep, zs + prng.gumbel(key, zs.shape), -np.inf)
+  srt = np.sort(noisy, axis=-1)
+  lead = srt[:, -1] - srt[:, -2] if k > 1 else np.full(len(z), np.inf)
+  return (gap > 8e-6) & ((lead > 1e-4) | ~np.isfinite(srt[:, -2])), keep.sum(axis=-1)
+
+
+@pytest.mark.parametrize('M,D,V,temp,top_p,top_k,sharp', [
+    (4, 256, 1024, 0.9, 0.9, None, 1.0), (64, 128, 4096, 1.0, 0.5, None, 4.0), (33, 256, 2080, 0.7, 1.0, 50, 1.0),
+    (5, 128, 2048, 1.0, 0.8, 100, 2.0), (128, 64, 8192, 1.0, 0.95, None, 1.0), (3, 128, 1024, 1.3, 0.3, 7, 8.0)])
+def test_head_nucleus_matches_oracle(M, D, V, temp, top_p, top_k, sharp):
+  x, w = _head_inputs(M, D, V, V + M)
+  w = bf16_round(w * sharp)
+  w[7], w[300] = w[3], w[3]  # equal logits: candidates tie, lower index ranks first
+  seed_key = prng.prng_key(77)
+  step = 4
+  _, _, _, logits = _run_head(x, w, 1, temp, seed_key, step)
+  tok, lp, _ = _run_nucleus(x, w, temp, top_p, top_k, seed_key, step)
+  key = prng.fold_in(seed_key, step)
+  want_tok, want_lp = OS.sample_top_p(logits, key, temp, top_p, top_k)
+  z = (logits / np.float32(temp)).astype(np.float32)
+  clear, nkeep = _nucleus_clear_rows(z, key, top_p, top_k)
+  assert clear.mean() > 0.6
+  np.testing.assert_array_equal(tok[clear, step + 1], want_tok[clear])
+  np.testing.assert_allclose(lp[clear, step + 1], want_lp[clear], atol=3e-5)
+  # every row: the token is a member of the oracle's nucleus (or sits exactly at the cut)
+  full_lp = OS.log_softmax(z)
+  np.testing.assert_allclose(lp[:, step + 1], full_lp[np.arange(M), tok[:, step + 1]], atol=3e-5)
+  for b in range(M):
+    if clear[b]:
+      members = OS.nucleus_members(z[b], top_p)
+      if top_k:
+        members &= set(np.argsort(-z[b], kind='stable')[:top_k].tolist())
+      assert int(tok[b, step + 1]) in members
+  assert np.all(tok[:, :step + 1] == -5) and np.all(tok[:, step + 2:] == -5)
+
+
+def test_head_nucleus_limits():
+  x, w = _head_inputs(16, 128, 1024, 3)
+  key = prng.prng_key(5)
+  _, _, _, logits = _run_head(x, w, 1, 1.0, key, 2)
+  # top_p -> 0 keeps only the best candidate: the draw is the argmax
+  tok, lp, _ = _run_nucleus(x, w, 1.0, 0.0, None, key, 2)
+  np.testing.assert_array_equal(tok[:, 3], np.argmax(logits, axis=-1))
+  # top_k = 1 likewise
+  tok1, _, _ = _run_nucleus(x, w, 1.0, 1.0, 1, key, 2)
+  np.testing.assert_array_equal(tok1[:, 3], np.argmax(logits, axis=-1))
+  # forbidden ids are never drawn and set no eos flag; eos flag follows the token
+  banned = tuple(int(t) for t in np.argsort(-logits[0])[:40])
+  tokf, lpf, done = _run_nucleus(x, w, 1.0, 0.9, None, key, 2, forbidden=banned, eos=(int(tok[0, 3]),))
+  assert not np.isin(tokf[:, 3], banned).any() and np.isfinite(lpf[:, 3]).all()
+  np.testing.assert_array_equal(done, (tokf[:, 3] == tok[0, 3]).astype(np.uint8))
+
+
+def test_head_nucleus_distribution_chi2():
+  # one sharp row repeated: empirical frequencies follow softmax(z) renormalised over the nucleus
+  M, D, V, top_p = 128, 128, 1024, 0.9
+  x, w = _head_inputs(1, D, V, 77)
+  w *= 5
+  x = np.repeat(x, M, axis=0)
+  counts = np.zeros(V)
+  _, _, _, logits = _run_head(x, w, 1, 1.0, prng.prng_key(5), 0)
+  for s in range(16):
+    tok, _, _ = _run_nucleus(x, w, 1.0, top_p, None, prng.prng_key(5), s)
+    counts += np.bincount(tok[:, s + 1], minlength=V)
+  members = sorted(OS.nucleus_members(logits[0], top_p))
+  assert counts.sum() == counts[members].sum()
+  pr = OS.softmax(logits[:1])[0].astype(np.float64)
+  pr = pr[members] / pr[members].sum()
+  assert len(members) > 7
+  top = np.argsort(-pr)[:6]
+  n = counts.sum()
+  obs = np.append(counts[members][top], n - counts[members][top].sum())
+  exp = np.append(pr[top], 1 - pr[top].sum()) * n
+  assert ((obs - exp) ** 2 / exp).sum() < 24.1  # 6 dof, p = 0.0005
+
+
 def test_head_sampling_distribution_chi2():
   T = G.Keep()
   # one sharp row repeated: empirical frequencies follow softmax(z)

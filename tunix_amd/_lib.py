@@ -28,6 +28,8 @@ SIGNATURES = {
     'tmx_gqa_decode_attention': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci],
     'tmx_head_sample': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
                         vp, vp],
+    'tmx_head_sample_nucleus': [vp, vp, vp, ci, ci, ci, cf, cf, ci, cu32, cu32, vp, vp, ci, vp, ci, vp, vp,
+                                vp, ci, vp, vp, ctypes.c_size_t],
     'tmx_decode_steps': [vp, vp, vp, ci, ci],
     'tmx_decode_steps_profiled': [vp, vp, vp, ci, ci, vp, vp],
 }
@@ -36,6 +38,7 @@ SIZE_FUNCS = {
     'tmx_gqa_decode_workspace_bytes': [ci, ci, ci, ci, ci],
     'tmx_qlora_linear_workspace_bytes': [ci, ci, ci],
     'tmx_head_sample_workspace_bytes': [ci, ci],
+    'tmx_nucleus_workspace_bytes': [ci, ci],
     'tmx_decode_workspace_bytes': [vp, ci, ci],
 }
 

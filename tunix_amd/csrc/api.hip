@@ -12,4 +12,4 @@ extern "C" const char* tmx_status_string(int status) {
   }
 }
 
-extern "C" int tmx_abi_version(void) { return 1; }
+extern "C" int tmx_abi_version(void) { return 2; }

@@ -101,8 +101,8 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   if (m->num_experts > 0) return TMX_ERR_UNSUPPORTED;
   const int B = s->batch, C = s->cache_size, L = s->buf_len;
   if (B <= 0 || B > 128 || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
-  if (sample && s->sampling_mode == TMX_SAMPLE_TOP_P && (s->top_p < 1.0f || s->top_k > 0))
-    return TMX_ERR_UNSUPPORTED;
+  const bool nucleus = sample && s->sampling_mode == TMX_SAMPLE_TOP_P && (s->top_p < 1.0f || s->top_k > 0);
+  if (nucleus && !s->nucleus_workspace) return TMX_ERR_ARG;
   const int D = m->embed_dim, N = m->num_heads, Kh = m->num_kv_heads, H = m->head_dim;
   const int F = m->hidden_dim, NH = N * H, QKV = (N + 2 * Kh) * H;
   if (carve(m, B, C, nullptr).total > s->workspace_bytes) return TMX_ERR_SHAPE;
@@ -248,7 +248,12 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       a.done = s->done;
       a.eos = s->eos_ids; a.n_eos = s->n_eos;
       a.buf_len = L;
-      TMX_TRY(TMX_K_HEAD, head_sample(st, a));
+      if (nucleus) {
+        TMX_TRY(TMX_K_HEAD, head_sample_nucleus(st, a, s->top_p, s->top_k, s->nucleus_workspace,
+                                                s->nucleus_workspace_bytes));
+      } else {
+        TMX_TRY(TMX_K_HEAD, head_sample(st, a));
+      }
     }
     TMX_TRY(TMX_K_ADVANCE, advance_step(st, s->step));
   }

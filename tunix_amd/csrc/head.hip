@@ -20,55 +20,9 @@
 // of ONE sequence: max / sum-exp / arg-best run down the registers without
 // cross-lane traffic.  Workgroup partials are merged by a second tiny kernel.
 #include "tmx_kernels.h"
+#include "tmx_sampling.h"
 
 namespace tmx {
-
-__device__ __forceinline__ uint32_t rotl32(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
-
-__device__ __forceinline__ void threefry2x32(uint32_t k0, uint32_t k1, uint32_t c0, uint32_t c1,
-                                             uint32_t& o0, uint32_t& o1) {
-  const uint32_t ks[3] = {k0, k1, k0 ^ k1 ^ 0x1BD11BDAu};
-  uint32_t x0 = c0 + ks[0], x1 = c1 + ks[1];
-  const int rot[2][4] = {{13, 15, 26, 6}, {17, 29, 16, 24}};
-#pragma unroll
-  for (int g = 0; g < 5; ++g) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      x0 += x1;
-      x1 = rotl32(x1, rot[g & 1][i]);
-      x1 ^= x0;
-    }
-    x0 += ks[(g + 1) % 3];
-    x1 += ks[(g + 2) % 3] + (uint32_t)(g + 1);
-  }
-  o0 = x0;
-  o1 = x1;
-}
-
-__device__ __forceinline__ float gumbel_from_bits(uint32_t bits) {
-  const float tiny = 1.17549435e-38f;
-  float f = __uint_as_float((bits >> 9) | 0x3F800000u) - 1.0f;
-  f = fmaxf(tiny, f + tiny);
-  return -logf(-logf(f));
-}
-
-struct Best {
-  float key;  // z + gumbel (or raw logit for greedy)
-  float z;
-  int idx;
-};
-__device__ __forceinline__ void best_merge(Best& a, const Best& b) {
-  if (b.key > a.key || (b.key == a.key && b.idx < a.idx)) a = b;
-}
-// (mx, se) <- merge with (mx2, se2): running max and sum of exp(z - max)
-__device__ __forceinline__ void lse_merge(float& mx, float& se, float mx2, float se2) {
-  const float mn = fmaxf(mx, mx2);
-  se = se * expf(mx - mn) + se2 * expf(mx2 - mn);
-  mx = mn;
-}
-
-
-constexpr float kNegBig = -3.0e38f;
 
 template <int V>
 struct HIC { static constexpr int value = V; };
@@ -191,9 +145,17 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
         float z = logit, key = logit;
         if (a.mode == TMX_SAMPLE_TOP_P) {
           z = logit / a.temperature;
-          uint32_t o0, o1;
-          threefry2x32(key0, key1, 0u, (uint32_t)row * (uint32_t)a.V + (uint32_t)v, o0, o1);
-          key = z + gumbel_from_bits(o0 ^ o1);
+          if (a.sort_keys) {
+            // ascending key order = descending z (with -0 == +0), rows kept apart by the high word
+            const uint32_t zb = __float_as_uint(z + 0.0f);
+            const uint32_t ord = (zb & 0x80000000u) ? ~zb : (zb | 0x80000000u);
+            a.sort_keys[(size_t)row * a.V + v] = ((uint64_t)row << 32) | (uint32_t)~ord;
+            key = z;
+          } else {
+            uint32_t o0, o1;
+            threefry2x32(key0, key1, 0u, (uint32_t)row * (uint32_t)a.V + (uint32_t)v, o0, o1);
+            key = z + gumbel_from_bits(o0 ^ o1);
+          }
         }
         if (z > mx) {
           se = se * expf(mx - z) + 1.f;
@@ -282,13 +244,17 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
   }
 }
 
-int head_sample(hipStream_t st, HeadArgs a) {
+int head_logits(hipStream_t st, HeadArgs& a) {
   if (a.V % 32 || a.D % 64 || a.M <= 0 || a.M > 128) return TMX_ERR_SHAPE;
   a.nwg = (a.V + 127) / 128;
   if (a.M <= 32) hipLaunchKernelGGL(head_kernel<1>, dim3(a.nwg), dim3(256), 0, st, a);
   else if (a.M <= 64) hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, a);
   else hipLaunchKernelGGL(head_kernel<4>, dim3(a.nwg), dim3(256), 0, st, a);
-  int rc = check_launch();
+  return check_launch();
+}
+
+int head_sample(hipStream_t st, HeadArgs a) {
+  int rc = head_logits(st, a);
   if (rc != TMX_OK) return rc;
   hipLaunchKernelGGL(head_finalize_kernel, dim3(a.M), dim3(256), 0, st, a);
   return check_launch();

@@ -103,6 +103,7 @@ struct HeadArgs {
   const int32_t* forbidden;
   int n_forbidden;
   float* logits_out;  // [M, V] raw f32 logits, optional
+  uint64_t* sort_keys;  // [M, V] (row << 32) | ~ordered(z): set for the sorting (nucleus / top-k) branch
   float* part_f;      // [M][nwg][4] = max, sumexp, best key, best z
   int32_t* part_i;    // [M][nwg]
   int nwg;
@@ -116,6 +117,23 @@ struct HeadArgs {
 };
 
 
+struct NucleusArgs {
+  const uint64_t* keys;  // [M, V] sorted ascending
+  const uint32_t* vals;  // [M, V] linear index row * V + v of each sorted key
+  int M, V, k;           // k: candidates kept by top-k (V without top-k)
+  float top_p;
+  uint32_t k0, k1;
+  const int32_t* step;
+  const float* part_f;   // head partials [M][nwg][4]
+  int nwg;
+  int32_t* token_buffer;
+  float* logprobs;
+  uint8_t* done;
+  const int32_t* eos;
+  int n_eos;
+  int buf_len;
+};
+
 int row_norm(hipStream_t st, const RowNormArgs& a, int M);
 int rope_kvwrite(hipStream_t st, const RopeArgs& a, int B);
 int swiglu(hipStream_t st, const SwigluArgs& a, int M);
@@ -124,6 +142,9 @@ int empty_launch(hipStream_t st);  // measurement aid: a kernel that does nothin
 int gqa_decode(hipStream_t st, AttnArgs a, int H);
 size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
 int head_sample(hipStream_t st, HeadArgs a);
+int head_logits(hipStream_t st, HeadArgs& a);  // the vocabulary kernel alone; fills a.nwg
+int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void* ws, size_t ws_bytes);
+size_t nucleus_bytes(int M, int V);
 size_t head_partial_bytes(int M, int V);
 int qlinear_num_splits(int K, int N, int M);
 int qlinear_num_lora_splits(int K);

@@ -89,7 +89,8 @@ class DecodeState(ctypes.Structure):
               ('seed_hi', ctypes.c_uint32), ('seed_lo', ctypes.c_uint32), ('eos_ids', ctypes.c_void_p),
               ('n_eos', ctypes.c_int), ('forbidden', ctypes.c_void_p), ('n_forbidden', ctypes.c_int),
               ('logits_out', ctypes.c_void_p), ('workspace', ctypes.c_void_p),
-              ('workspace_bytes', ctypes.c_size_t)]
+              ('workspace_bytes', ctypes.c_size_t), ('nucleus_workspace', ctypes.c_void_p),
+              ('nucleus_workspace_bytes', ctypes.c_size_t)]
 
 
 def _qdesc(pl):

@@ -88,6 +88,7 @@ class Sampler:
     self._lib = _lib.lib()  # raises if the HIP library is missing
     self._cache = None
     self._workspace = None
+    self._nucleus_ws = None
     self.eos_ids = None
     self.last_step_logits = None
 
@@ -206,6 +207,14 @@ class Sampler:
       s.forbidden, s.n_forbidden = st['forbidden'].data_ptr(), st['forbidden'].numel()
     s.logits_out = st['logits'].data_ptr() if st['logits'] is not None else None
     s.workspace, s.workspace_bytes = self._workspace.data_ptr(), self._workspace.numel()
+    if s.sampling_mode == SAMPLE_TOP_P and (s.top_p < 1.0 or s.top_k > 0):
+      # the sorting branch of sample_top_p needs room for one sort key per logit
+      nb = self._lib.tmx_nucleus_workspace_bytes(b, self._transformer.config.vocab_size)
+      if nb == 0:
+        raise _lib.TmxError('tmx_nucleus_workspace_bytes returned 0 (no device, or batch x vocab too large)')
+      if self._nucleus_ws is None or self._nucleus_ws.numel() < nb:
+        self._nucleus_ws = torch.empty(nb, dtype=torch.uint8, device=self._transformer.device)
+      s.nucleus_workspace, s.nucleus_workspace_bytes = self._nucleus_ws.data_ptr(), self._nucleus_ws.numel()
     return s
 
   def run_steps(self, st, n_steps, sample=True):
