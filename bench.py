@@ -247,7 +247,7 @@ def main():
     # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
     mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
     symbols = {
-        f'tmx::qlinear_mfma_kernel<{mt}>': ['qkv_linear', 'o_linear', 'gate_up_linear', 'down_linear'],
+        f'tmx::qlinear_mfma_kernel<{mt}, *>': ['qkv_linear', 'o_linear', 'gate_up_linear', 'down_linear'],
         f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention'],
         f'tmx::head_kernel<{mt}>': ['head_sample'],
     }

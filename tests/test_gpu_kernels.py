@@ -73,7 +73,9 @@ def test_qlora_linear_matches_oracle(M, K, N, group, r):
     # f32 accumulation order differs: at most one bf16 ulp of the base projection (which the
     # LoRA / residual adds can turn into several ulps of a small sum), and only rarely
     base = bf16_round(x @ lin.weight())
-    G.assert_bf16_close(G.host(y), ref, ulps=1.0, extra=G.ulp_bf16(base) if (use_res or r) else 0.0,
+    # a one-ulp flip of the base or of base + LoRA (before the residual is added) carries through
+    extra = np.maximum(G.ulp_bf16(base), G.ulp_bf16(out)) if (use_res or r) else 0.0
+    G.assert_bf16_close(G.host(y), ref, ulps=1.0, extra=extra,
                         min_exact=0.995, what=f'linear {M}x{K}x{N}')
 
 

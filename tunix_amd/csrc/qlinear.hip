@@ -41,6 +41,21 @@ __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s)
 }
 
 
+template <int V>
+struct IC { static constexpr int value = V; };
+
+// f(IC<0>{}), ..., f(IC<N - 1>{}): a loop whose index is a compile-time constant
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(IC<I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
+// Two kernels share the tile math.  The 4-wave kernel (one wave per column tile, steps of 4
+// k-tiles) serves K % 256 == 0 below 8192; the k-way kernel further down runs two waves per
+// column tile over steps of 8 k-tiles, takes any K % 64 == 0 and serves the deep projections.
 // One workgroup = 4 waves owns a block of 4 adjacent 32-column tiles (one per wave) over one
 // K-slice and advances in steps of KS = 4 k-tiles (256 k).  Per step the activation slab
 // x[0:M, 256 s : 256 s + 256] is fetched once per workgroup with coalesced 16-byte loads
@@ -53,14 +68,11 @@ __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s)
 constexpr int kKS = 4;                    // k-tiles per pipeline step
 constexpr int kXStride = kKS * 64 + 8;    // bf16 elements per LDS row
 
-template <int V>
-struct IC { static constexpr int value = V; };
-
 // LORA = false: one int4 column tile per wave.  LORA = true: the block computes a K-slice
 // of t = x . A from bf16 tiles of A (one 32-column tile per wave); A is stored in MFMA
 // B-fragment order, [K/64][Rpad/32][64 lanes][4 steps][8], so a wave reads 4 KiB contiguously.
 template <int MT, bool LORA>
-__device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[MT * 32][kXStride]) {
+__device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)[MT * 32][kXStride]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = lane >> 5, nl = lane & 31;
   const int KT = a.K >> 6;
@@ -210,28 +222,255 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t (*xs)[
 }
 
 template <int MT>
-__global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void qlinear_mfma_kernel(QLinearArgs a) {
+__global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void qlinear_mfma4_kernel(QLinearArgs a) {
   __shared__ __align__(16) uint16_t xs[2][MT * 32][kXStride];
-  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block<MT, true>(a, xs);
-  else gemm_block<MT, false>(a, xs);
+  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block4<MT, true>(a, xs);
+  else gemm_block4<MT, false>(a, xs);
 }
 
 template <int MT>
-static int launch_qlinear(hipStream_t st, QLinearArgs a) {
+static int launch_qlinear4(hipStream_t st, QLinearArgs a) {
   a.n_main_blocks = (a.N + 127) / 128;
   const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
-  hipLaunchKernelGGL((qlinear_mfma_kernel<MT>), dim3(blocks, a.nsplit), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((qlinear_mfma4_kernel<MT>), dim3(blocks, a.nsplit), dim3(256), 0, st, a);
   return check_launch();
 }
+
+// One workgroup owns a block of 4 adjacent 32-column tiles over one K-slice.  It runs 4 * KW
+// waves: wave (ct, kw) multiplies column tile ct by every KW-th group of TPW k-tiles, so a CU
+// holds 2-4 waves per SIMD whose dequantisation (VALU), MFMA and load latencies overlap.  The
+// workgroup advances in steps of KS k-tiles: the activation slab x[0:M, step] is fetched once
+// with coalesced 16-byte loads (issued one step ahead), double-buffered in LDS (rows padded by
+// 16 bytes: conflict-free ds_read_b128) and shared by all waves as MFMA A fragments; weights go
+// HBM -> registers through a ring that keeps two steps in flight per wave.  The KW partial
+// accumulators of a column tile are added through LDS at the end.  Small-N projections are also
+// split along K over blockIdx.y so that every CU streams weights; each split writes its own f32
+// plane (summed by the consumer kernel), so results do not depend on scheduling order.
+template <int MT, int KW_>
+struct Shape {
+  static constexpr int KW = KW_;                // k-ways: waves sharing one column tile
+  static constexpr int KS = (MT == 4 || KW_ == 1) ? 4 : 8;  // k-tiles per step
+  static constexpr int TPW = KS / KW;           // k-tiles per wave and step
+  static constexpr int NTHR = 256 * KW;
+  static constexpr int ROWS = MT * 32;
+  static constexpr int XS = KS * 64 + 8;        // bf16 elements per LDS row
+  static constexpr size_t LDS = (size_t)2 * ROWS * XS * 2;
+};
+
+// LORA = false: int4 column tiles.  LORA = true: the block computes a K-slice of t = x . A from
+// bf16 tiles of A; A is stored in MFMA B-fragment order, [K/64][Rpad/32][64 lanes][4 steps][8],
+// so a wave reads the 4 KiB of a tile contiguously.
+template <int MT, int KW_, bool LORA>
+__device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t* smem) {
+  using S = Shape<MT, KW_>;
+  constexpr int KW = S::KW, KS = S::KS, TPW = S::TPW, NTHR = S::NTHR, ROWS = S::ROWS, XS = S::XS;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ct = wave & 3, kw = wave >> 2;
+  const int h = lane >> 5, nl = lane & 31;
+  const int KT = a.K >> 6;
+  // K-slice of this block: main blocks follow blockIdx.y; the LoRA blocks of a launch cut K
+  // into finer slices of their own so that none of them is the last to finish
+  const int slice = LORA ? ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y
+                         : (int)blockIdx.y;
+  const int per = LORA ? a.kt_per_lora_split : a.kt_per_split;
+  const int kb0 = slice * per;
+  const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
+  const int ntiles = kb1 - kb0;
+  if (ntiles <= 0) return;
+  const int nsteps = (ntiles + KS - 1) / KS;
+  const int kpg_shift = (a.G == 64) ? 0 : __builtin_ctz(a.G >> 6), KG = a.K / a.G;
+
+  // this wave's column tile; waves past the last tile idle through the steps
+  const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
+  const int nb = LORA ? ct : (int)blockIdx.x * 4 + ct;
+  const bool tile_ok = nb < NT;
+
+  f32x16_t acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
+
+  // cooperative activation load: chunk c = tid + NTHR i -> row c / CPR, 16-byte column c % CPR
+  constexpr int CPR = KS * 8;
+  constexpr int XC = ROWS * CPR / NTHR;
+  const uint16_t* xsrc[XC];
+  int xoff_l[XC], xmax[XC];
+#pragma unroll
+  for (int i = 0; i < XC; ++i) {
+    const int c = tid + NTHR * i;
+    const int row_l = c / CPR, col_l = (c % CPR) * 8;
+    xoff_l[i] = row_l * XS + col_l;
+    const int row = row_l < a.M ? row_l : a.M - 1;
+    xsrc[i] = a.x + (size_t)row * a.ldx + (size_t)kb0 * 64 + col_l;
+    xmax[i] = a.K - 8 - (kb0 * 64 + col_l);  // last in-bounds offset (columns of skipped tiles)
+  }
+  constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
+  constexpr int DW = LORA ? 1 : 2;   // steps of weights in flight
+  const u32x4_t* wsrc = nullptr;
+  const uint16_t* ssrc = nullptr;
+  size_t wstep = 0;  // 16-byte words between consecutive k-tiles of one column tile
+  if (tile_ok) {
+    if (LORA) {
+      wstep = (size_t)NT * 64 * 4;
+      wsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + ((size_t)nb * 64 + lane) * 4 + (size_t)kb0 * wstep;
+    } else {
+      wstep = 64;
+      wsrc = reinterpret_cast<const u32x4_t*>(a.qw) + (size_t)nb * KT * 64 + lane + (size_t)kb0 * wstep;
+      ssrc = a.scales + (size_t)nb * KG * 32 + nl;
+    }
+  }
+  u32x4_t xreg[XC];
+  u32x4_t wring[DW][TPW][WPT];
+  uint16_t sring[DW][TPW];
+  const int last_step = nsteps - 1, last_tile = ntiles - 1;
+
+  // Unconditional loads with clamped indices: the compiler can then count the outstanding
+  // loads exactly and wait only for the oldest one.
+  auto load_w_tile = [&](int step, auto dc, auto jc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+    step = step < last_step ? step : last_step;
+    int rel = step * KS + kw * TPW + j;  // k-tile relative to kb0
+    rel = rel < last_tile ? rel : last_tile;
+#pragma unroll
+    for (int t = 0; t < WPT; ++t) wring[d][j][t] = wsrc[(size_t)rel * wstep + t];
+    if (!LORA) sring[d][j] = ssrc[(size_t)((kb0 + rel) >> kpg_shift) * 32];
+  };
+  auto load_w = [&](int step, auto dc) __attribute__((always_inline)) {
+    static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(step, dc, jc); });
+  };
+  auto load_x = [&](int step) __attribute__((always_inline)) {
+    step = step < last_step ? step : last_step;
+#pragma unroll
+    for (int i = 0; i < XC; ++i) {
+      int off = step * KS * 64;
+      off = off < xmax[i] ? off : xmax[i];
+      xreg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + off);
+    }
+  };
+  auto stash_x = [&](int buf) __attribute__((always_inline)) {
+    uint16_t* base = smem + (size_t)buf * ROWS * XS;
+#pragma unroll
+    for (int i = 0; i < XC; ++i) *reinterpret_cast<u32x4_t*>(base + xoff_l[i]) = xreg[i];
+  };
+  // one k-tile of this wave
+  auto tile_math = [&](int step, int buf, auto dc, auto jc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kw * TPW + j) * 64 + h * 8;
+    bf16x8_t xa[MT][4];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + (m * 32 + nl) * XS + t * 16);
+    u32x4_t wc[WPT];
+#pragma unroll
+    for (int t = 0; t < WPT; ++t) wc[t] = wring[d][j][t];
+    const float s_c = LORA ? 0.f : bf2f(sring[d][j]);
+    load_w_tile(step + DW, dc, jc);  // slot consumed: refill it DW steps ahead
+    if (step * KS + kw * TPW + j > last_tile) return;  // past the slice (ragged last step)
+    const float m8s = -8.f * s_c;
+    const uint32_t wd[4] = {wc[0].x, wc[0].y, wc[0].z, wc[0].w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      bf16x8_t b;
+      if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[t % WPT]);
+      else b = dequant_word(wd[t], s_c, m8s);
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[m], 0, 0, 0);
+    }
+  };
+  // step s: activations in LDS buffer s & 1, weights in ring slot s % DW
+  auto do_step = [&](int step, auto sc) __attribute__((always_inline)) {
+    constexpr int sp = decltype(sc)::value;  // step parity (static)
+    constexpr int d = sp % DW;
+    load_x(step + 1);
+    if (tile_ok)
+      static_for<TPW>([&](auto jc) __attribute__((always_inline)) { tile_math(step, sp, IC<d>{}, jc); });
+    stash_x(sp ^ 1);
+    __syncthreads();
+  };
+
+  load_x(0);
+  if (tile_ok) {
+    load_w(0, IC<0>{});
+    if (DW == 2) load_w(1, IC<1 % DW>{});
+  }
+  stash_x(0);
+  __syncthreads();
+  const int npairs = nsteps / 2;
+  for (int g = 0; g < npairs; ++g) {
+    do_step(2 * g, IC<0>{});
+    do_step(2 * g + 1, IC<1>{});
+  }
+  if (nsteps & 1) do_step(nsteps - 1, IC<0>{});
+
+  // add the KW partial accumulators of each column tile through LDS (the slab is free now: the
+  // last step ended with a barrier); layout [kw - 1][ct][m][r][lane] keeps every access linear
+  float* red = reinterpret_cast<float*>(smem);
+  if (kw > 0) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        red[(((((kw - 1) * 4 + ct) * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
+  }
+  if (KW > 1) __syncthreads();
+  if (kw > 0 || !tile_ok) return;
+#pragma unroll
+  for (int k = 1; k < KW; ++k)
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[m][r] += red[(((((k - 1) * 4 + ct) * MT + m) * 16 + r) << 6) + lane];
+
+  const int col = nb * 32 + nl;
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = m * 32 + acc_row(r, lane);
+      if (row >= a.M) continue;
+      if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = acc[m][r];
+      else if (a.y_bf16) a.y_bf16[(size_t)row * a.N + col] = f2bf(acc[m][r]);
+      else a.y_part[((size_t)slice * a.M + row) * a.N + col] = acc[m][r];
+    }
+}
+
+template <int MT, int KW>
+__global__ __launch_bounds__((Shape<MT, KW>::NTHR), 1) void qlinear_mfma_kernel(QLinearArgs a) {
+  extern __shared__ __align__(16) uint16_t smem[];
+  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block<MT, KW, true>(a, smem);
+  else gemm_block<MT, KW, false>(a, smem);
+}
+
+template <int MT, int KW>
+static int launch_qlinear(hipStream_t st, QLinearArgs a) {
+  using S = Shape<MT, KW>;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&qlinear_mfma_kernel<MT, KW>), hipFuncAttributeMaxDynamicSharedMemorySize,
+      (int)S::LDS);
+  if (attr != hipSuccess) return TMX_ERR_LAUNCH;
+  a.n_main_blocks = (a.N + 127) / 128;
+  const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
+  hipLaunchKernelGGL((qlinear_mfma_kernel<MT, KW>), dim3(blocks, a.nsplit), dim3(S::NTHR), S::LDS, st, a);
+  return check_launch();
+}
+
+static bool four_wave(int K) { return K % 256 == 0 && K < 8192; }
 
 static int slice_len(int KT, int s) { return ((KT + s - 1) / s + 3) / 4 * 4; }
 static bool slices_ok(int KT, int s) { return (KT + slice_len(KT, s) - 1) / slice_len(KT, s) == s; }
 
+// Number of K-slices for a projection: the count that minimises (rounds of workgroups over the
+// 256 CUs) x (steps per slice + fixed start-up / reduction work), with a small charge per plane
+// for the f32 traffic of the partial sums.  No slice may be empty.
 // Number of K-slices for a projection.  Wide projections (>= 192 column blocks) are not
 // split: they write bf16 directly.  Otherwise the smallest power of two that gives at least
 // 128 workgroups and at most 32 k-tiles per slice, in whole groups of 4 k-tiles, no empty slice.
-int qlinear_num_splits(int K, int N, int M) {
-  (void)M;
+static int num_splits4(int K, int N) {
   const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
   if (nblocks >= 192) return 1;
@@ -244,14 +483,38 @@ int qlinear_num_splits(int K, int N, int M) {
   return best;
 }
 
-// Number of K-slices of the LoRA projection t = x . A: as fine as whole groups of 4 k-tiles
-// allow (at most TMX_MAX_LORA_SPLITS planes), so that no LoRA block outlasts the main blocks.
-int qlinear_num_lora_splits(int K) {
+int qlinear_num_splits(int K, int N, int M) {
+  if (four_wave(K)) return num_splits4(K, N);
+  const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
-  for (int per = 4;; per += 4) {
+  const int ks = M > 64 ? 4 : 8;
+  int best = 1;
+  float best_cost = 1e30f;
+  for (int s = 1; s <= TMX_MAX_SPLITS; ++s) {
+    if (!slices_ok(KT, s)) continue;
+    const int rounds = (nblocks * s + 255) / 256;
+    const int nsteps = (slice_len(KT, s) + ks - 1) / ks;
+    const float cost = rounds * (nsteps + 2.0f) + 0.15f * s;
+    if (cost < best_cost) { best_cost = cost; best = s; }
+  }
+  return best;
+}
+
+// Number of K-slices of the LoRA projection t = x . A: as fine as whole steps (4 or 8 k-tiles,
+// by kernel) allow, at most TMX_MAX_LORA_SPLITS planes, so that no LoRA block outlasts the
+// main blocks.
+static int lora_step(int K) { return four_wave(K) ? 4 : 8; }
+int qlinear_num_lora_splits(int K) {
+  const int KT = K / 64, g = lora_step(K);
+  for (int per = g;; per += g) {
     const int n = (KT + per - 1) / per;
     if (n <= TMX_MAX_LORA_SPLITS) return n;
   }
+}
+
+static int lora_slice_len(int K) {
+  const int KT = K / 64, n = qlinear_num_lora_splits(K), g = lora_step(K);
+  return ((KT + n - 1) / n + g - 1) / g * g;
 }
 
 // Host-side dispatch shared by the C entry point and the decode-step launcher.
@@ -262,7 +525,7 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
                  int N, int G, int Rpad, int nsplit) {
   if (!x || !qw || !scales || (!y_bf16 && !y_part)) return TMX_ERR_ARG;
   if (M <= 0 || M > 128 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
-  if (K % 256 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
+  if (K % 64 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
   if (a_t && (!t_part || Rpad <= 0 || Rpad % 32 || Rpad > 128 || ldt < Rpad)) return TMX_ERR_SHAPE;
   if (nsplit < 1 || nsplit > TMX_MAX_SPLITS || (nsplit > 1 && !y_part)) return TMX_ERR_ARG;
   const int KT = K / 64;
@@ -282,10 +545,15 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   a.kt_per_split = slice_len(KT, nsplit);
   const int nls = qlinear_num_lora_splits(K);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
-  a.kt_per_lora_split = slice_len(KT, nls);
-  if (M <= 32) return launch_qlinear<1>(st, a);
-  if (M <= 64) return launch_qlinear<2>(st, a);
-  return launch_qlinear<4>(st, a);
+  a.kt_per_lora_split = lora_slice_len(K);
+  if (four_wave(K)) {
+    if (M <= 32) return launch_qlinear4<1>(st, a);
+    if (M <= 64) return launch_qlinear4<2>(st, a);
+    return launch_qlinear4<4>(st, a);
+  }
+  if (M <= 32) return launch_qlinear<1, 2>(st, a);
+  if (M <= 64) return launch_qlinear<2, 2>(st, a);
+  return launch_qlinear<4, 2>(st, a);
 }
 
 // ---------------------------------------------------------------------------
