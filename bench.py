@@ -24,15 +24,20 @@ WORKLOADS = {
     'llama3.1-8b-grpo': ('llama3p1_8b', 64, 256, 512, 64, 16, 0.9, 1.0),
     'llama3.2-1b-b1': ('llama3p2_1b', 1, 256, 512, 64, 16, 1.0, 1.0),
     'toy': ('toy', 4, 32, 32, 64, 8, 0.9, 1.0),
+    # large-batch rollout with nucleus sampling, and the MoE shape (LoRA on attention only)
+    'qwen3-8b-b128': ('qwen3_8b', 128, 512, 1024, 128, 32, 1.0, 0.95),
+    'qwen3-30b-a3b-moe': ('qwen3_30b_a3b', 32, 256, 512, 64, 8, 0.9, 1.0),
 }
+ATTN_ONLY_LORA = {'qwen3-30b-a3b-moe'}
 
 CLASS_NAMES = ['row_norm', 'qkv_linear', 'rope_kvwrite', 'attention', 'o_linear', 'gate_up_linear',
-               'swiglu', 'down_linear', 'head_sample', 'advance_step', 'empty_launch']
+               'swiglu', 'down_linear', 'head_sample', 'advance_step', 'empty_launch', 'router']
 
 
-def linear_bytes(pl, batch):
-  """int4 + scales + LoRA A, B (+ activations in and out, counted for the GEMM regime)."""
-  b = pl.k * pl.n // 2 + (pl.k // pl.group) * pl.n * 2
+def linear_bytes(pl, batch, frac=1.0):
+  """int4 + scales + LoRA A, B (+ activations in and out, counted for the GEMM regime).
+  frac: expected fraction of a stacked expert matrix that a step touches."""
+  b = int((pl.k * pl.n // 2 + (pl.k // pl.group) * pl.n * 2) * (frac if pl.experts > 1 else 1.0))
   if pl.lora_a_t is not None:
     b += 2 * pl.rank * (pl.k * len(pl.seg_cols) + pl.n)
   return b + batch * (pl.k + pl.n) * 2
@@ -128,7 +133,11 @@ def main():
     sys.exit(2)
   cfg = getattr(ModelConfig, name)()
   torch.cuda.set_device(0)
-  model = QLoRAModel.random_init(cfg, seed=0, group=group, lora_rank=rank, lora_alpha=2.0 * rank)
+  targets = ('q_proj', 'k_proj', 'v_proj', 'o_proj')
+  if args.workload not in ATTN_ONLY_LORA:
+    targets += ('gate_proj', 'up_proj', 'down_proj')
+  model = QLoRAModel.random_init(cfg, seed=0, group=group, lora_rank=rank, lora_alpha=2.0 * rank,
+                                 lora_targets=targets)
   cache_size = prompt + new
 
   class _Tok:  # ids only: the benchmark feeds token ids and never decodes text
@@ -141,7 +150,8 @@ def main():
   sampler = Sampler(model, _Tok(), CacheConfig(cache_size, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
   sampler.eos_ids = np.array([-1])  # unreachable: every row runs the full length
   rng = np.random.default_rng(0)
-  n_prompts = max(batch // 8, 1)
+  # GRPO workloads: G = 8 samples of a prompt are consecutive rows; the others: distinct prompts
+  n_prompts = max(batch // 8, 1) if 'grpo' in args.workload else batch
   base = rng.integers(3, cfg.vocab_size, (n_prompts, prompt)).astype(np.int32)
   ids = np.repeat(base, batch // n_prompts, axis=0)  # G samples of a prompt are consecutive rows
 
@@ -199,7 +209,7 @@ def main():
   }
 
   # Whole-step algorithmic bytes at the mean context of the timed region.
-  wbytes, hbytes = model.weight_bytes()
+  wbytes, hbytes = model.weight_bytes(batch)
   s_mean = prompt + args.warmup + args.steps / 2.0
   kv_per_tok = cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * 2 * 2
   step_bytes = wbytes + hbytes + batch * s_mean * kv_per_tok
@@ -239,18 +249,29 @@ def main():
     ctx = ctx_sum / max(ctx_n, 1)
     alg = {
         'qkv_linear': linear_bytes(layer0['qkv'], batch), 'o_linear': linear_bytes(layer0['o'], batch),
-        'gate_up_linear': linear_bytes(layer0['gate_up'], batch),
-        'down_linear': linear_bytes(layer0['down'], batch),
+        'gate_up_linear': linear_bytes(layer0['gate_up'], batch, model.expert_fraction(batch)),
+        'down_linear': linear_bytes(layer0['down'], batch, model.expert_fraction(batch)),
         'attention': batch * ctx * cfg.num_kv_heads * cfg.head_dim * 2 * 2,
         'head_sample': hbytes,
     }
     # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
     mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
-    symbols = {
-        f'tmx::qlinear_mfma_kernel<{mt}, *>': ['qkv_linear', 'o_linear', 'gate_up_linear', 'down_linear'],
+    # projections with K % 256 == 0 below 8192 run the 4-wave kernel, deeper ones the k-way kernel
+    four = lambda pl: pl.k % 256 == 0 and pl.k < 8192
+    dense = [('qkv_linear', 'qkv'), ('o_linear', 'o')]
+    symbols = {}
+    if cfg.num_experts:
+      symbols['tmx::moe_expert_kernel<false>'] = ['gate_up_linear']
+      symbols['tmx::moe_expert_kernel<true>'] = ['down_linear']
+    else:
+      dense += [('gate_up_linear', 'gate_up'), ('down_linear', 'down')]
+    for cls_name, key in dense:
+      sym = f'tmx::qlinear_mfma4_kernel<{mt}>' if four(layer0[key]) else f'tmx::qlinear_mfma_kernel<{mt}, 2>'
+      symbols.setdefault(sym, []).append(cls_name)
+    symbols.update({
         f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention'],
         f'tmx::head_kernel<{mt}>': ['head_sample'],
-    }
+    })
     idx = {n: i for i, n in enumerate(CLASS_NAMES)}
     # An event pair around a launch also times the packet processing on both sides of it, so it
     # reads a few microseconds above rocprofv3's kernel trace (which brackets the dispatch
@@ -283,7 +304,7 @@ def main():
                           'algorithmic_bytes_per_launch': d['algorithmic_bytes_per_launch'],
                           'note': 'mean HIP-event time around the launches of this kernel in the sampled '
                                   'steps (includes event packet processing, see empty_launch_event_pair_ms); '
-                                  'the projection kernel serves qkv, o, gate|up and down'}
+                                  'the 4-wave projection kernel serves qkv, o and gate|up, the k-way kernel down'}
     result['roofline_kernels'] = per_symbol
     result['roofline_all'] = {}
     for i, n in enumerate(CLASS_NAMES):
@@ -292,7 +313,7 @@ def main():
         result['roofline_all'][n] = {'avg_launch_ms': avg, 'achieved_GBps': alg[n] / (avg * 1e-3) / 1e9,
                                      'frac': alg[n] / (avg * 1e-3) / 8e12}
 
-  if not args.no_cpu_baseline:
+  if not args.no_cpu_baseline and not cfg.num_experts:
     del st
     result['cpu_baseline'] = cpu_baseline(args.workload)
   print(json.dumps(result))

@@ -165,6 +165,25 @@ int tmx_head_sample_nucleus(void* stream, const void* x, const void* head_w, int
                             float* logprobs, uint8_t* done, int buf_len, void* workspace,
                             void* nucleus_workspace, size_t nucleus_workspace_bytes);
 
+/* ---- routed experts (Qwen3 MoE) ----------------------------------------------- */
+
+/* Routing of tunix/models/qwen3/model.py:895-902: scores = bf16(x[B, D] . router_w[D, E]),
+ * f32 softmax, top_k (ties: lower expert id), weights renormalised over the top_k and rounded
+ * to bf16.  expert_of / weight_of: [B, top_k]. */
+int tmx_moe_route(void* stream, const void* x, const void* router_w, int B, int D, int E, int top_k,
+                  int32_t* expert_of, float* weight_of);
+
+/* One launch over all experts (the routed pairs of tunix/models/qwen3/model.py:911-939):
+ * pair p = token * top_k + slot belongs to expert expert_of[p]; experts nobody routed to are
+ * not read.  qweight / scales: E stacked per-expert matrices [K, N] in the q4t / scale layout.
+ *   down == 0: x = hidden states [P / top_k, K = D] (row p / top_k), N = 2 F with columns
+ *              gate | up; out[p, 0:F] = bf16(silu(gate) * up) (F % 64 == 0)
+ *   down != 0: x = activations [P, K = F] (row p); out[p, 0:N] = bf16(x . W_e) (N % 128 == 0)
+ * K % 256 == 0, P <= 1024. */
+int tmx_moe_experts(void* stream, const void* x, int ldx, const void* qweight, const void* scales,
+                    const int32_t* expert_of, int P, int top_k, int E, int K, int N, int G, int down,
+                    void* out, int ldo);
+
 /* ---- whole decode steps ------------------------------------------------------ */
 
 
@@ -184,8 +203,9 @@ typedef struct {
   const void* k_norm_w;
   tmx_qlinear_desc qkv;     /* columns: q (N H) | k (Kh H) | v (Kh H) */
   tmx_qlinear_desc o;       /* [N H, D] */
-  tmx_qlinear_desc gate_up; /* columns: gate (F) | up (F) */
-  tmx_qlinear_desc down;    /* [F, D] */
+  tmx_qlinear_desc gate_up; /* columns: gate (F) | up (F); MoE: num_experts such matrices stacked */
+  tmx_qlinear_desc down;    /* [F, D]; MoE: num_experts stacked */
+  const void* router_w;     /* MoE: bf16 [D, num_experts] router kernel, else NULL */
 } tmx_layer_desc;
 
 typedef struct {
@@ -253,7 +273,8 @@ int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state,
 #define TMX_K_HEAD 8     /* head + log-softmax + token selection (+ finalize) */
 #define TMX_K_ADVANCE 9
 #define TMX_K_EMPTY 10   /* one empty launch per layer: what an event pair costs by itself */
-#define TMX_NUM_KERNEL_CLASSES 11
+#define TMX_K_ROUTER 11  /* MoE router: scores, softmax, top-k */
+#define TMX_NUM_KERNEL_CLASSES 12
 int tmx_decode_steps_profiled(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
                               int n_steps, int sample, float* class_ms_host, int* class_launches_host);
 

@@ -54,6 +54,12 @@ def make_state(cfg, seed=0, lora_rank=0, targets=('q_proj', 'k_proj', 'v_proj', 
     if cfg.family == 'qwen3':
       st[f'{p}.attn.q_norm.w'] = ones(h)
       st[f'{p}.attn.k_norm.w'] = ones(h)
+    if cfg.num_experts:
+      e = cfg.num_experts
+      st[f'{p}.mlp.router.kernel'] = mat(d, e) * np.float32(8)  # spread-out routing scores
+      st[f'{p}.mlp.gate_proj'], st[f'{p}.mlp.up_proj'] = mat(e, d, f), mat(e, d, f)
+      st[f'{p}.mlp.down_proj'] = mat(e, f, d)
+      continue
     for name, (k, o) in {'gate_proj': (d, f), 'up_proj': (d, f), 'down_proj': (f, d)}.items():
       st[f'{p}.mlp.{name}.kernel'] = mat(k, o)
       if lora_rank and name in targets:
@@ -83,9 +89,18 @@ def oracle_weights(cfg, st, group, lora_alpha, lora_rank, quantized=True):
     p = f'layers.{i}'
     lw = {'norm1': st[f'{p}.input_layernorm.w'], 'norm2': st[f'{p}.post_attention_layernorm.w'],
           'q': lin(f'{p}.attn', 'q_proj', 'w'), 'k': lin(f'{p}.attn', 'k_proj', 'w'),
-          'v': lin(f'{p}.attn', 'v_proj', 'w'), 'o': lin(f'{p}.attn', 'o_proj', 'w'),
-          'gate': lin(f'{p}.mlp', 'gate_proj', 'kernel'), 'up': lin(f'{p}.mlp', 'up_proj', 'kernel'),
-          'down': lin(f'{p}.mlp', 'down_proj', 'kernel')}
+          'v': lin(f'{p}.attn', 'v_proj', 'w'), 'o': lin(f'{p}.attn', 'o_proj', 'w')}
+    if cfg.num_experts:
+      def elin(w2):
+        q, s = int4.quantize(w2, group)
+        return OL.Linear(q=q, scale=s, group=group)
+      lw['router'] = st[f'{p}.mlp.router.kernel']
+      lw['experts'] = [(elin(st[f'{p}.mlp.gate_proj'][e]), elin(st[f'{p}.mlp.up_proj'][e]),
+                        elin(st[f'{p}.mlp.down_proj'][e])) for e in range(cfg.num_experts)]
+    else:
+      lw['gate'] = lin(f'{p}.mlp', 'gate_proj', 'kernel')
+      lw['up'] = lin(f'{p}.mlp', 'up_proj', 'kernel')
+      lw['down'] = lin(f'{p}.mlp', 'down_proj', 'kernel')
     if cfg.family == 'qwen3':
       lw['q_norm'], lw['k_norm'] = st[f'{p}.attn.q_norm.w'], st[f'{p}.attn.k_norm.w']
     w['layers'].append(lw)
@@ -95,7 +110,8 @@ def oracle_weights(cfg, st, group, lora_alpha, lora_rank, quantized=True):
 def product_config(cfg):
   from tunix_amd.model import ModelConfig
   return ModelConfig(cfg.family, cfg.num_layers, cfg.vocab_size, cfg.embed_dim, cfg.hidden_dim,
-                     cfg.num_heads, cfg.head_dim, cfg.num_kv_heads, cfg.rope_theta, cfg.norm_eps, cfg.tied)
+                     cfg.num_heads, cfg.head_dim, cfg.num_kv_heads, cfg.rope_theta, cfg.norm_eps, cfg.tied,
+                     cfg.num_experts or None, cfg.experts_per_tok or None)
 
 
 def product_model(cfg, st, group, lora_alpha, device='cuda'):

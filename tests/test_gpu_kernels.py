@@ -457,3 +457,74 @@ def test_head_sampling_distribution_chi2():
   obs = np.append(counts[top], n - counts[top].sum())
   exp = np.append(pr[top], 1 - pr[top].sum()) * n
   assert ((obs - exp) ** 2 / exp).sum() < 27.9  # 8 dof, p = 0.0005
+
+
+# ---- routed experts (Qwen3 MoE) ---------------------------------------------------------------
+
+@pytest.mark.parametrize('B,D,E,k', [(8, 256, 16, 4), (32, 512, 128, 8), (3, 256, 8, 1)])
+def test_moe_route_matches_oracle(B, D, E, k):
+  T = G.Keep()
+  rng = np.random.default_rng(B + E)
+  x = bf16_round(rng.standard_normal((B, D)).astype(np.float32))
+  rw = bf16_round(rng.standard_normal((D, E)).astype(np.float32) * 0.2)
+  idx = torch.full((B, k), -1, dtype=torch.int32, device=G.DEV)
+  wt = torch.zeros(B, k, dtype=torch.float32, device=G.DEV)
+  G.call('tmx_moe_route', S(), T.bf(x), T.bf(rw), B, D, E, k, G.p(idx), G.p(wt))
+  G.sync()
+  want_w, want_idx = L.moe_route(x, rw, k)
+  # expert sets are compared where the k-th / (k+1)-th score margin is clear of bf16 rounding
+  scores = np.sort(bf16_round(x @ rw), axis=-1)[:, ::-1]
+  clear = np.ones(B, bool) if k == E else (scores[:, k - 1] - scores[:, k]) > 2 * G.ulp_bf16(scores[:, k - 1])
+  ordered = np.all(np.diff(scores[:, :k], axis=-1) < -2 * G.ulp_bf16(scores[:, :1]), axis=-1) if k > 1 else clear
+  assert clear.mean() > 0.5
+  got_idx, got_w = idx.cpu().numpy(), wt.cpu().numpy()
+  for b in range(B):
+    if clear[b]:
+      assert set(got_idx[b]) == set(want_idx[b])
+    if clear[b] and ordered[b]:
+      np.testing.assert_array_equal(got_idx[b], want_idx[b])
+      np.testing.assert_allclose(got_w[b], want_w[b], atol=2 * G.ulp_bf16(want_w[b]).max())
+  np.testing.assert_allclose(got_w.sum(-1), 1.0, atol=0.02)
+  assert (got_idx >= 0).all() and (got_idx < E).all()
+  assert all(len(set(r)) == k for r in got_idx)
+
+
+@pytest.mark.parametrize('B,D,F,E,k,group', [(8, 256, 256, 16, 4, 64), (32, 512, 256, 32, 8, 128), (40, 256, 512, 4, 2, 64)])
+def test_moe_experts_match_oracle(B, D, F, E, k, group):
+  T = G.Keep()
+  rng = np.random.default_rng(B * 3 + E)
+  x = bf16_round(rng.standard_normal((B, D)).astype(np.float32))
+  gate = bf16_round(rng.standard_normal((E, D, F)).astype(np.float32) * 0.05)
+  up = bf16_round(rng.standard_normal((E, D, F)).astype(np.float32) * 0.05)
+  down = bf16_round(rng.standard_normal((E, F, D)).astype(np.float32) * 0.05)
+  # routing table: every token picks k distinct experts; expert E - 1 is never used; when the
+  # batch allows it one expert receives more than 32 rows (second row chunk)
+  idx = np.stack([rng.permutation(E - 1)[:k] for _ in range(B)]).astype(np.int32)
+  if B > 32:
+    idx[:, 0] = 0
+  gu = np.stack([gate, up], axis=2).transpose(1, 0, 2, 3).reshape(D, E * 2 * F)
+  dn = down.transpose(1, 0, 2).reshape(F, E * D)
+  pgu, pdn = _packed(gu, group), _packed(dn, group)
+  P = B * k
+  idx_t = T.i32(idx.reshape(-1))
+  act = torch.full((P, F), 7.0, dtype=torch.bfloat16, device=G.DEV)
+  y = torch.full((P, D), 7.0, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_moe_experts', S(), T.bf(x), D, G.p(pgu.qweight), G.p(pgu.scales), idx_t, P, k, E, D, 2 * F,
+         group, 0, G.p(act), F)
+  G.call('tmx_moe_experts', S(), G.p(act), F, G.p(pdn.qweight), G.p(pdn.scales), idx_t, P, k, E, F, D,
+         group, 1, G.p(y), D)
+  G.sync()
+  got_act, got_y = G.host(act), G.host(y)
+  lin = lambda w: L.Linear(q=int4.quantize(w, group)[0], scale=int4.quantize(w, group)[1], group=group)
+  for e in range(E - 1):
+    rows = np.nonzero(idx.reshape(-1) == e)[0]
+    if rows.size == 0:
+      continue
+    xe = x[rows // k]
+    g, u = lin(gate[e])(xe, BF16), lin(up[e])(xe, BF16)
+    want_act = bf16_round(L.silu(g, BF16) * u)
+    # a one-ulp flip of g or u (f32 accumulation order) moves the product by about one ulp of it
+    G.assert_bf16_close(got_act[rows], want_act, ulps=2.0, extra=1e-6, min_exact=0.98, what=f'act e{e}')
+    want_y = lin(down[e])(got_act[rows], BF16)  # the kernel's own activations: isolates the down product
+    G.assert_bf16_close(got_y[rows], want_y, ulps=1.0, min_exact=0.995, what=f'down e{e}')
+  assert not np.isin(idx, E - 1).any()

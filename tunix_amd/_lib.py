@@ -30,6 +30,8 @@ SIGNATURES = {
                         vp, vp],
     'tmx_head_sample_nucleus': [vp, vp, vp, ci, ci, ci, cf, cf, ci, cu32, cu32, vp, vp, ci, vp, ci, vp, vp,
                                 vp, ci, vp, vp, ctypes.c_size_t],
+    'tmx_moe_route': [vp, vp, vp, ci, ci, ci, ci, vp, vp],
+    'tmx_moe_experts': [vp, vp, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, vp, ci],
     'tmx_decode_steps': [vp, vp, vp, ci, ci],
     'tmx_decode_steps_profiled': [vp, vp, vp, ci, ci, vp, vp],
 }

@@ -52,8 +52,11 @@ __global__ __launch_bounds__(AttnWaves<G>::value * 64) void gqa_decode_kernel(At
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int pg = lane / LPP, dl = lane % LPP;  // lane group, 8-element slice index
   const int step = *a.step;
-  const int s_begin = split * a.chunk;
-  int s_end = s_begin + a.chunk;
+  // the splits share the VALID positions 0 .. step (not the cache size) in chunks of whole
+  // 32 positions, so that every split has work at any context length
+  const int chunk = (((step + a.nsplit) / a.nsplit) + 31) & ~31;
+  const int s_begin = split * chunk;
+  int s_end = s_begin + chunk;
   if (s_end > step + 1) s_end = step + 1;
 
   // query fragments for the G heads of this kv head: 8 bf16 = 4 packed pairs each
@@ -211,7 +214,6 @@ size_t attn_partial_bytes(int B, int N, int Kh, int H, int C) {
 
 int gqa_decode(hipStream_t st, AttnArgs a, int H) {
   a.nsplit = attn_num_splits(a.B, a.Kh, a.C);
-  a.chunk = (a.C + a.nsplit - 1) / a.nsplit;
   if (a.nsplit > 1 && !a.partial) return TMX_ERR_ARG;
   const int G = a.N / a.Kh;
   if (a.N % a.Kh) return TMX_ERR_SHAPE;

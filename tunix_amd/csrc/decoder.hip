@@ -21,6 +21,10 @@ struct Workspace {
   float *y_part, *t_part, *rope_tab;
   float* attn_partial;
   void* head_partial;
+  // routed experts (MoE models)
+  int32_t* expert_of;
+  float* weight_of;
+  uint16_t *pair_act, *pair_y;
   size_t total;
 };
 
@@ -32,8 +36,8 @@ static Splits plan_splits(const tmx_model_desc* m, int B) {
   Splits s;
   s.qkv = qlinear_num_splits(D, QKV, B);
   s.o = qlinear_num_splits(NH, D, B);
-  s.gate_up = qlinear_num_splits(D, 2 * F, B);
-  s.down = qlinear_num_splits(F, D, B);
+  s.gate_up = m->num_experts > 0 ? 1 : qlinear_num_splits(D, 2 * F, B);
+  s.down = m->num_experts > 0 ? 1 : qlinear_num_splits(F, D, B);
   return s;
 }
 
@@ -59,6 +63,11 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   w.rope_tab = (float*)take((size_t)B * m->head_dim * 4);
   w.attn_partial = (float*)take(attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C));
   w.head_partial = take(head_partial_bytes(B, m->vocab_size));
+  const size_t P = m->num_experts > 0 ? (size_t)B * m->experts_per_tok : 0;
+  w.expert_of = (int32_t*)take(P * 4);
+  w.weight_of = (float*)take(P * 4);
+  w.pair_act = (uint16_t*)take(P * F * 2);
+  w.pair_y = (uint16_t*)take(P * D * 2);
   w.total = off;
   return w;
 }
@@ -98,7 +107,10 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   if (!s->token_buffer || !s->positions || !s->input_mask || !s->done || !s->step || !s->kv_cache ||
       !s->workspace)
     return TMX_ERR_ARG;
-  if (m->num_experts > 0) return TMX_ERR_UNSUPPORTED;
+  const bool moe = m->num_experts > 0;
+  if (moe && (m->experts_per_tok <= 0 || m->experts_per_tok > m->num_experts ||
+              (size_t)s->batch * m->experts_per_tok > 1024))
+    return TMX_ERR_SHAPE;
   const int B = s->batch, C = s->cache_size, L = s->buf_len;
   if (B <= 0 || B > 128 || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
   const bool nucleus = sample && s->sampling_mode == TMX_SAMPLE_TOP_P && (s->top_p < 1.0f || s->top_k > 0);
@@ -110,9 +122,12 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     const tmx_layer_desc& l = m->layers[i];
     if (!l.norm1_w || !l.norm2_w) return TMX_ERR_ARG;
     int rc;
-    if ((rc = check_linear(l.qkv, D, QKV)) || (rc = check_linear(l.o, NH, D)) ||
-        (rc = check_linear(l.gate_up, D, 2 * F)) || (rc = check_linear(l.down, F, D)))
-      return rc;
+    if ((rc = check_linear(l.qkv, D, QKV)) || (rc = check_linear(l.o, NH, D))) return rc;
+    if (moe) {
+      if (!l.router_w || l.gate_up.lora_a_t || l.down.lora_a_t) return TMX_ERR_ARG;
+    }
+    // dense: one matrix; MoE: num_experts stacked matrices of the same per-expert shape
+    if ((rc = check_linear(l.gate_up, D, 2 * F)) || (rc = check_linear(l.down, F, D))) return rc;
   }
   hipStream_t st = (hipStream_t)stream;
   const Workspace w = carve(m, B, C, (char*)s->workspace);
@@ -199,33 +214,66 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
         TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
       }
-      const bool gu16 = sp.gate_up == 1;
-      TMX_TRY(TMX_K_GATE_UP, qlinear_base(st, w.xn, D, l.gate_up.qweight, l.gate_up.scales,
-                                          l.gate_up.lora_a_t, gu16 ? w.y16 : nullptr, w.y_part, w.t_part,
-                                          TMX_MAX_RPAD, B, D, 2 * F, l.gate_up.G, l.gate_up.r_pad,
-                                          sp.gate_up));
-      {
-        SwigluArgs a = {};
-        a.gu_bf16 = gu16 ? w.y16 : nullptr;
-        a.gu_part = w.y_part;
-        a.nsplit = sp.gate_up;
-        a.lora = lora_of(l.gate_up, sp.gate_up);
-        a.act = w.act; a.F = F;
-        TMX_TRY(TMX_K_SWIGLU, swiglu(st, a, B));
-      }
-      TMX_TRY(TMX_K_DOWN, qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t,
-                                       nullptr, w.y_part, w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G,
-                                       l.down.r_pad, sp.down));
-      {
+      if (moe) {
+        const int P = B * m->experts_per_tok;
+        {
+          RouterArgs a = {};
+          a.x = w.xn;
+          a.w = (const uint16_t*)l.router_w;
+          a.D = D; a.E = m->num_experts; a.top_k = m->experts_per_tok;
+          a.expert_of = w.expert_of; a.weight_of = w.weight_of;
+          TMX_TRY(TMX_K_ROUTER, moe_route(st, a, B));
+        }
+        MoeArgs e = {};
+        e.expert_of = w.expert_of; e.P = P; e.top_k = m->experts_per_tok;
+        e.x = w.xn; e.ldx = D;
+        e.qw = (const uint4*)l.gate_up.qweight; e.scales = (const uint16_t*)l.gate_up.scales;
+        e.K = D; e.N = 2 * F; e.G = l.gate_up.G;
+        e.qw_stride = (size_t)e.K * e.N / 32; e.sc_stride = (size_t)(e.K / e.G) * e.N;
+        e.out = w.pair_act; e.ldo = F;
+        TMX_TRY(TMX_K_GATE_UP, moe_experts(st, e, m->num_experts, false));
+        e.x = w.pair_act; e.ldx = F;
+        e.qw = (const uint4*)l.down.qweight; e.scales = (const uint16_t*)l.down.scales;
+        e.K = F; e.N = D; e.G = l.down.G;
+        e.qw_stride = (size_t)e.K * e.N / 32; e.sc_stride = (size_t)(e.K / e.G) * e.N;
+        e.out = w.pair_y; e.ldo = D;
+        TMX_TRY(TMX_K_DOWN, moe_experts(st, e, m->num_experts, true));
         RowNormArgs a = {};
-        a.y_part = w.y_part;
-        a.nsplit = sp.down;
-        a.lora = lora_of(l.down, sp.down);
+        a.moe_y = w.pair_y; a.moe_w = w.weight_of; a.top_k = m->experts_per_tok;
         a.residual = w.x; a.x_out = w.x;
         a.norm_w = (const uint16_t*)(i + 1 < m->num_layers ? m->layers[i + 1].norm1_w : m->final_norm_w);
         a.xn_out = w.xn;
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
         TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
+      } else {
+        const bool gu16 = sp.gate_up == 1;
+        TMX_TRY(TMX_K_GATE_UP, qlinear_base(st, w.xn, D, l.gate_up.qweight, l.gate_up.scales,
+                                            l.gate_up.lora_a_t, gu16 ? w.y16 : nullptr, w.y_part, w.t_part,
+                                            TMX_MAX_RPAD, B, D, 2 * F, l.gate_up.G, l.gate_up.r_pad,
+                                            sp.gate_up));
+        {
+          SwigluArgs a = {};
+          a.gu_bf16 = gu16 ? w.y16 : nullptr;
+          a.gu_part = w.y_part;
+          a.nsplit = sp.gate_up;
+          a.lora = lora_of(l.gate_up, sp.gate_up);
+          a.act = w.act; a.F = F;
+          TMX_TRY(TMX_K_SWIGLU, swiglu(st, a, B));
+        }
+        TMX_TRY(TMX_K_DOWN, qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t,
+                                         nullptr, w.y_part, w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G,
+                                         l.down.r_pad, sp.down));
+        {
+          RowNormArgs a = {};
+          a.y_part = w.y_part;
+          a.nsplit = sp.down;
+          a.lora = lora_of(l.down, sp.down);
+          a.residual = w.x; a.x_out = w.x;
+          a.norm_w = (const uint16_t*)(i + 1 < m->num_layers ? m->layers[i + 1].norm1_w : m->final_norm_w);
+          a.xn_out = w.xn;
+          a.D = D; a.eps = m->norm_eps; a.family = m->family;
+          TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
+        }
       }
       if (prof) TMX_TRY(TMX_K_EMPTY, empty_launch(st));
     }

@@ -168,6 +168,19 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
       const int n0 = c * 8;
       if (src) {
         unpack8(*reinterpret_cast<const uint4*>(src + n0), v[i]);
+      } else if (a.moe_y) {
+        // bf16(sum over the token's experts of weight * expert output), f32 accumulation
+        for (int j = 0; j < a.top_k; ++j) {
+          float y8[8];
+          const size_t p = (size_t)m * a.top_k + j;
+          unpack8(*reinterpret_cast<const uint4*>(a.moe_y + p * a.D + n0), y8);
+          const float w = a.moe_w[p];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[i][e] = fmaf(w, y8[e], v[i][e]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e]);
+        if (a.residual) unpack8(*reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0), res8[i]);
       } else {
         load_base8(a.y_bf16, a.y_part, a.nsplit, m, M, a.D, n0, v[i]);
         if (a.residual) unpack8(*reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0), res8[i]);

@@ -79,7 +79,7 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
   // K-slice of this block: main blocks follow blockIdx.y; the LoRA blocks of a launch cut K
   // into finer slices of their own so that none of them is the last to finish
   const int slice = LORA ? ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y
-                         : (int)blockIdx.y;
+                         : (a.fixed_slice >= 0 ? a.fixed_slice : (int)blockIdx.y);
   const int per = LORA ? a.kt_per_lora_split : a.kt_per_split;
   const int kb0 = slice * per;
   const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
@@ -89,7 +89,10 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
 
   // this wave's column tile; waves past the last tile recompute the last one (result dropped)
   const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
-  const int nb_mine = LORA ? wave : (int)blockIdx.x * 4 + wave;
+  // pair mode: waves 0, 1 take two gate tiles, waves 2, 3 the matching up tiles
+  const int nb_mine = LORA ? wave
+                      : a.pair_off ? (int)blockIdx.x * 2 + (wave & 1) + (wave >> 1) * a.pair_off
+                                   : (int)blockIdx.x * 4 + wave;
   const bool tile_ok = nb_mine < NT;
   const int nb = tile_ok ? nb_mine : NT - 1;
 
@@ -108,7 +111,8 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
     const int c = tid + 256 * i;
     const int row_l = c >> 5, col_l = (c & 31) * 8;
     xoff_l[i] = row_l * kXStride + col_l;
-    const int row = row_l < a.M ? row_l : a.M - 1;
+    int row = row_l < a.M ? row_l : a.M - 1;
+    if (a.row_src) row = a.row_src[row];
     xsrc[i] = a.x + (size_t)row * a.ldx + (size_t)kb0 * 64 + col_l;
   }
   constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
@@ -205,6 +209,33 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
   }
   if (nsteps & 1) do_step(nsteps - 1, IC<0>{});
 
+  if (!LORA && a.pair_off) {
+    // act = bf16(bf16(g * bf16(sigmoid(g))) * u), g / u = bf16 gate / up projections: the up
+    // waves hand their tile to the gate waves through LDS (the slab is free after the last barrier)
+    float* ex = reinterpret_cast<float*>(&xs[0][0][0]);  // [2][MT][16][64]
+    if (wave >= 2) {
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ex[((((wave - 2) * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
+    }
+    __syncthreads();
+    if (wave < 2 && tile_ok) {
+      const int col = ((int)blockIdx.x * 2 + wave) * 32 + nl;
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m * 32 + acc_row(r, lane);
+          if (row >= a.M) continue;
+          const float g = rbf(acc[m][r]), u = rbf(ex[(((wave * MT + m) * 16 + r) << 6) + lane]);
+          const float sg = rbf(1.f / (1.f + expf(-g)));
+          const int drow = a.row_dst ? a.row_dst[row] : row;
+          a.y_bf16[(size_t)drow * a.ldy + col] = f2bf(rbf(g * sg) * u);
+        }
+    }
+    return;
+  }
   // epilogue: every wave owns its tile outright
   if (tile_ok) {
     const int col = nb_mine * 32 + nl;
@@ -214,8 +245,9 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
       for (int r = 0; r < 16; ++r) {
         const int row = m * 32 + acc_row(r, lane);
         if (row >= a.M) continue;
+        const int drow = (!LORA && a.row_dst) ? a.row_dst[row] : row;
         if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = acc[m][r];
-        else if (a.y_bf16) a.y_bf16[(size_t)row * a.N + col] = f2bf(acc[m][r]);
+        else if (a.y_bf16) a.y_bf16[(size_t)drow * a.ldy + col] = f2bf(acc[m][r]);
         else a.y_part[((size_t)slice * a.M + row) * a.N + col] = acc[m][r];
       }
   }
@@ -233,6 +265,79 @@ static int launch_qlinear4(hipStream_t st, QLinearArgs a) {
   a.n_main_blocks = (a.N + 127) / 128;
   const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
   hipLaunchKernelGGL((qlinear_mfma4_kernel<MT>), dim3(blocks, a.nsplit), dim3(256), 0, st, a);
+  return check_launch();
+}
+
+// Routed experts: grid (column blocks, experts).  Every workgroup first collects the pairs
+// (token, slot) routed to its expert from the routing table (at most a few hundred entries),
+// leaves if there are none (so unrouted experts are never streamed), and otherwise runs the
+// 4-wave block over its rows in chunks of 32 with gathered activation rows and scattered
+// output rows.  DOWN = false fuses SwiGLU: the workgroup owns 64 gate columns and the matching
+// 64 up columns.  tunix/models/qwen3/model.py:894-939 evaluated for routed pairs only.
+template <bool DOWN>
+__global__ __launch_bounds__(256, 2) void moe_expert_kernel(MoeArgs m) {
+  __shared__ __align__(16) uint16_t xs[2][32][kXStride];
+  __shared__ int rows_s[1024];
+  __shared__ int src_s[32], dst_s[32];
+  __shared__ int wave_cnt[4];
+  __shared__ int n_s;
+  const int e = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int base = 0;
+  for (int p0 = 0; p0 < m.P; p0 += 256) {  // ordered compaction of { p : expert_of[p] == e }
+    const int p = p0 + tid;
+    const bool hit = p < m.P && m.expert_of[p] == e;
+    const unsigned long long mask = __ballot(hit);
+    if (lane == 0) wave_cnt[wave] = __popcll(mask);
+    __syncthreads();
+    int off = base;
+    for (int w = 0; w < wave; ++w) off += wave_cnt[w];
+    if (hit) rows_s[off + __popcll(mask & ((1ull << lane) - 1ull))] = p;
+    base += wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
+    __syncthreads();
+  }
+  if (tid == 0) n_s = base;
+  __syncthreads();
+  const int n = n_s;
+  if (n == 0) return;
+  QLinearArgs a = {};
+  a.x = m.x;
+  a.ldx = m.ldx;
+  a.qw = m.qw + (size_t)e * m.qw_stride;
+  a.scales = m.scales + (size_t)e * m.sc_stride;
+  a.y_bf16 = m.out;
+  a.ldy = m.ldo;
+  a.K = m.K; a.N = m.N; a.G = m.G;
+  a.n_main_blocks = gridDim.x;
+  a.nsplit = 1;
+  a.kt_per_split = m.K >> 6;
+  a.fixed_slice = 0;
+  a.row_src = src_s;
+  a.row_dst = dst_s;
+  a.pair_off = DOWN ? 0 : (m.N >> 6);  // tiles in F = N / 2 columns
+  for (int c0 = 0; c0 < n; c0 += 32) {
+    if (tid < 32 && c0 + tid < n) {
+      const int p = rows_s[c0 + tid];
+      src_s[tid] = DOWN ? p : p / m.top_k;
+      dst_s[tid] = p;
+    }
+    __syncthreads();
+    a.M = n - c0 < 32 ? n - c0 : 32;
+    gemm_block4<1, false>(a, xs);
+    __syncthreads();
+  }
+}
+
+int moe_experts(hipStream_t st, const MoeArgs& a, int E, bool down) {
+  if (!a.x || !a.qw || !a.scales || !a.expert_of || !a.out) return TMX_ERR_ARG;
+  if (a.P <= 0 || a.P > 1024 || a.top_k <= 0 || E <= 0) return TMX_ERR_SHAPE;
+  if (a.K % 256 || a.G % 64 || (a.G & (a.G - 1)) || a.K % a.G || a.ldx % 8) return TMX_ERR_SHAPE;
+  if (down) {
+    if (a.N % 128) return TMX_ERR_SHAPE;
+    hipLaunchKernelGGL(moe_expert_kernel<true>, dim3(a.N / 128, E), dim3(256), 0, st, a);
+  } else {
+    if (a.N % 128) return TMX_ERR_SHAPE;  // F % 64 == 0
+    hipLaunchKernelGGL(moe_expert_kernel<false>, dim3(a.N / 128, E), dim3(256), 0, st, a);
+  }
   return check_launch();
 }
 
@@ -434,7 +539,7 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t* smem)
       const int row = m * 32 + acc_row(r, lane);
       if (row >= a.M) continue;
       if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = acc[m][r];
-      else if (a.y_bf16) a.y_bf16[(size_t)row * a.N + col] = f2bf(acc[m][r]);
+      else if (a.y_bf16) a.y_bf16[(size_t)row * a.ldy + col] = f2bf(acc[m][r]);
       else a.y_part[((size_t)slice * a.M + row) * a.N + col] = acc[m][r];
     }
 }
@@ -530,7 +635,9 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   if (nsplit < 1 || nsplit > TMX_MAX_SPLITS || (nsplit > 1 && !y_part)) return TMX_ERR_ARG;
   const int KT = K / 64;
   if (!slices_ok(KT, nsplit)) return TMX_ERR_SHAPE;  // an empty K-slice
-  QLinearArgs a;
+  QLinearArgs a = {};
+  a.fixed_slice = -1;
+  a.ldy = N;
   a.x = (const uint16_t*)x;
   a.ldx = ldx;
   a.qw = (const uint4*)qw;

@@ -17,6 +17,34 @@ struct QLinearArgs {
   int M, K, N, G, Rpad;
   int n_main_blocks, nsplit, kt_per_split;
   int lora_blocks_per_split, kt_per_lora_split;  // finer K-slices of the LoRA projection
+  // routed-expert use of the 4-wave block (all zero / null / -1 for plain projections)
+  int ldy;                 // row stride of y_bf16
+  int fixed_slice;         // K-slice index when blockIdx.y means something else (-1: blockIdx.y)
+  const int* row_src;      // activation row of tile row i (null: i)
+  const int* row_dst;      // output row of tile row i (null: i)
+  int pair_off;            // != 0: gate | up pairing, tile distance between a gate tile and its up tile
+};
+
+// Routed experts (Qwen3 MoE): one launch multiplies, for every expert, the rows routed to it.
+struct MoeArgs {
+  const uint16_t* x;       // gate|up: normed hidden states [B, D]; down: activations [P, F]
+  int ldx;
+  const uint4* qw;         // [E] stacked q4t matrices
+  const uint16_t* scales;  // [E] stacked scale arrays
+  size_t qw_stride, sc_stride;  // elements between consecutive experts
+  const int32_t* expert_of;     // [P] expert of pair p = token * top_k + slot
+  int P, top_k;
+  int K, N, G;             // per-expert matrix [K, N] (gate|up: N = 2 F)
+  uint16_t* out;           // gate|up: act [P, F]; down: y [P, D]
+  int ldo;
+};
+
+struct RouterArgs {
+  const uint16_t* x;       // [B, D] normed hidden states
+  const uint16_t* w;       // [D, E] bf16 router kernel
+  int D, E, top_k;
+  int32_t* expert_of;      // [B, top_k]
+  float* weight_of;        // [B, top_k] renormalised routing weights (bf16 values)
 };
 
 // The LoRA-B half applied by the consumer of a projection.
@@ -42,6 +70,9 @@ struct RowNormArgs {
   const float* y_part;          // [nsplit][M][D] f32 planes
   int nsplit;
   LoraIn lora;
+  const uint16_t* moe_y;        // [M * top_k, D] routed-expert outputs (replaces y when set)
+  const float* moe_w;           // [M * top_k] routing weights
+  int top_k;
   const uint16_t* residual;     // [M, D] (null: none)
   uint16_t* x_out;              // [M, D] new residual stream (null: not stored)
   const uint16_t* norm_w;       // [D] (null: no norm output)
@@ -141,6 +172,8 @@ int advance_step(hipStream_t st, int32_t* step);
 int empty_launch(hipStream_t st);  // measurement aid: a kernel that does nothing
 int gqa_decode(hipStream_t st, AttnArgs a, int H);
 size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
+int moe_route(hipStream_t st, const RouterArgs& a, int B);
+int moe_experts(hipStream_t st, const MoeArgs& a, int E, bool down);
 int head_sample(hipStream_t st, HeadArgs a);
 int head_logits(hipStream_t st, HeadArgs& a);  // the vocabulary kernel alone; fills a.nwg
 int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void* ws, size_t ws_bytes);

@@ -68,7 +68,7 @@ class QLinearDesc(ctypes.Structure):
 class LayerDesc(ctypes.Structure):
   _fields_ = [('norm1_w', ctypes.c_void_p), ('norm2_w', ctypes.c_void_p), ('q_norm_w', ctypes.c_void_p),
               ('k_norm_w', ctypes.c_void_p), ('qkv', QLinearDesc), ('o', QLinearDesc),
-              ('gate_up', QLinearDesc), ('down', QLinearDesc)]
+              ('gate_up', QLinearDesc), ('down', QLinearDesc), ('router_w', ctypes.c_void_p)]
 
 
 class ModelDesc(ctypes.Structure):
@@ -98,7 +98,7 @@ def _qdesc(pl):
   d.qweight, d.scales = pl.qweight.data_ptr(), pl.scales.data_ptr()
   d.lora_a_t = pl.lora_a_t.data_ptr() if pl.lora_a_t is not None else None
   d.lora_b = pl.lora_b.data_ptr() if pl.lora_b is not None else None
-  d.K, d.N, d.G, d.rank, d.r_pad, d.lora_scale = pl.k, pl.n, pl.group, pl.rank, pl.r_pad, pl.lora_scale
+  d.K, d.N, d.G, d.rank, d.r_pad, d.lora_scale = pl.k, pl.n // pl.experts, pl.group, pl.rank, pl.r_pad, pl.lora_scale
   return d
 
 
@@ -144,8 +144,6 @@ class QLoRAModel:
     'layers.0.mlp.gate_proj.kernel' [D, F], '...kernel_lora_a', '...kernel_lora_b',
     'layers.0.input_layernorm.w', 'embedder.input_embedding' [V, D], 'final_norm.w',
     'lm_head.w' [D, V] (untied)."""
-    if config.num_experts:
-      raise NotImplementedError('MoE layers are not packed by this build yet')
     m = cls(config, device)
     m.group, m.lora_alpha = group, float(lora_alpha)
     dev = m.device
@@ -178,9 +176,21 @@ class QLoRAModel:
           'norm2': bf(state[f'{p}.post_attention_layernorm.w']),
           'qkv': proj(f'{p}.attn', ('q_proj', 'k_proj', 'v_proj'), 'w'),
           'o': proj(f'{p}.attn', ('o_proj',), 'w'),
-          'gate_up': proj(f'{p}.mlp', ('gate_proj', 'up_proj'), 'kernel'),
-          'down': proj(f'{p}.mlp', ('down_proj',), 'kernel'),
       }
+      if config.num_experts:
+        # MoELayer params (tunix/models/qwen3/model.py:863-891): router.kernel [D, E],
+        # gate_proj / up_proj [E, D, F], down_proj [E, F, D]; no LoRA on experts
+        e = config.num_experts
+        g_, u_ = (torch.as_tensor(state[f'{p}.mlp.{n}']).to(dev) for n in ('gate_proj', 'up_proj'))
+        gu = torch.stack([g_, u_], dim=2).permute(1, 0, 2, 3).reshape(g_.shape[1], -1)  # [D, E * (F | F)]
+        dn = torch.as_tensor(state[f'{p}.mlp.down_proj']).to(dev).permute(1, 0, 2).reshape(g_.shape[2], -1)
+        layer['gate_up'] = quant.PackedLinear.from_dense([gu], group, dev, None, 0.0, bound)
+        layer['down'] = quant.PackedLinear.from_dense([dn], group, dev, None, 0.0, bound)
+        layer['gate_up'].experts = layer['down'].experts = e
+        layer['router'] = bf(state[f'{p}.mlp.router.kernel'])
+      else:
+        layer['gate_up'] = proj(f'{p}.mlp', ('gate_proj', 'up_proj'), 'kernel')
+        layer['down'] = proj(f'{p}.mlp', ('down_proj',), 'kernel')
       if config.family == 'qwen3':
         layer['q_norm'] = bf(state[f'{p}.attn.q_norm.w'])
         layer['k_norm'] = bf(state[f'{p}.attn.k_norm.w'])
@@ -216,9 +226,16 @@ class QLoRAModel:
           'norm2': torch.ones(d, dtype=torch.bfloat16, device=device),
           'qkv': proj(d, (nh, kh, kh), ('q_proj', 'k_proj', 'v_proj')),
           'o': proj(nh, (d,), ('o_proj',)),
-          'gate_up': proj(d, (f, f), ('gate_proj', 'up_proj')),
-          'down': proj(f, (d,), ('down_proj',)),
       }
+      if c.num_experts:
+        e = c.num_experts
+        layer['gate_up'] = quant.PackedLinear.from_dense([rnd(d, e * 2 * f)], group, device)
+        layer['down'] = quant.PackedLinear.from_dense([rnd(f, e * d)], group, device)
+        layer['gate_up'].experts = layer['down'].experts = e
+        layer['router'] = rnd(d, e)
+      else:
+        layer['gate_up'] = proj(d, (f, f), ('gate_proj', 'up_proj'))
+        layer['down'] = proj(f, (d,), ('down_proj',))
       if c.family == 'qwen3':
         layer['q_norm'] = torch.ones(c.head_dim, dtype=torch.bfloat16, device=device)
         layer['k_norm'] = torch.ones(c.head_dim, dtype=torch.bfloat16, device=device)
@@ -305,6 +322,7 @@ class QLoRAModel:
       arr[i].k_norm_w = layer['k_norm'].data_ptr() if 'k_norm' in layer else None
       arr[i].qkv, arr[i].o = _qdesc(layer['qkv']), _qdesc(layer['o'])
       arr[i].gate_up, arr[i].down = _qdesc(layer['gate_up']), _qdesc(layer['down'])
+      arr[i].router_w = layer['router'].data_ptr() if 'router' in layer else None
     d = ModelDesc()
     d.family = FAMILY_LLAMA3 if c.family == 'llama3' else FAMILY_QWEN3
     d.num_layers, d.vocab_size, d.embed_dim, d.hidden_dim = c.num_layers, c.vocab_size, c.embed_dim, c.hidden_dim
@@ -316,14 +334,26 @@ class QLoRAModel:
     self._desc, self._keep = d, arr
     return d
 
-  def weight_bytes(self):
+  def expert_fraction(self, batch):
+    """Expected fraction of a layer's experts that a step of `batch` tokens touches under
+    uniform routing: 1 - (1 - k / E) ** batch (1 for dense models)."""
+    c = self.config
+    if not c.num_experts:
+      return 1.0
+    return 1.0 - (1.0 - c.num_experts_per_tok / c.num_experts) ** batch
+
+  def weight_bytes(self, batch=1):
     """Algorithmic bytes one decode step streams from the weights:
-    int4 + scales + LoRA A, B per projection, plus the bf16 head."""
+    int4 + scales + LoRA A, B per projection, plus the bf16 head.  Routed-expert
+    matrices count by the expected fraction of experts touched (data dependent)."""
     total = 0
     for layer in self.layers:
+      if 'router' in layer:
+        total += layer['router'].numel() * 2
       for key in ('qkv', 'o', 'gate_up', 'down'):
         pl = layer[key]
-        total += pl.k * pl.n // 2 + (pl.k // pl.group) * pl.n * 2
+        frac = self.expert_fraction(batch) if pl.experts > 1 else 1.0
+        total += int((pl.k * pl.n // 2 + (pl.k // pl.group) * pl.n * 2) * frac)
         if pl.lora_a_t is not None:
           total += 2 * pl.rank * (pl.k * len(pl.seg_cols) + pl.n)
     return total, self.head.numel() * 2

@@ -78,6 +78,10 @@ class PackedLinear:
     self.seg_cols = list(seg_cols)
     self.rank = rank
     self.lora_a_t, self.lora_b, self.lora_scale = lora_a_t, lora_b, float(lora_scale)
+    # > 1: `n` columns hold that many equally wide per-expert matrices side by side; a tile
+    # column never straddles experts, so expert e's q4t tiles and scales are one contiguous
+    # slice (the stacked layout the routed-expert kernel reads)
+    self.experts = 1
 
   @property
   def r_pad(self):
