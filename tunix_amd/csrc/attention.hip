@@ -197,7 +197,8 @@ static int launch_attn(hipStream_t st, const AttnArgs& a) {
   return check_launch();
 }
 
-// Number of sequence splits that brings the grid to roughly two workgroups per CU.
+// Number of sequence splits that brings the grid to roughly two workgroups per CU (more splits
+// cost more in partial sums and the combine launch than they gain at rollout batch sizes).
 int attn_num_splits(int B, int Kh, int C) {
   int ns = 512 / (B * Kh);
   if (ns < 1) ns = 1;

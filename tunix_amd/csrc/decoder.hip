@@ -174,6 +174,9 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     }
     for (int i = 0; i < m->num_layers; ++i) {
       const tmx_layer_desc& l = m->layers[i];
+      // gate | up with LoRA + SwiGLU in its epilogue: 4-wave kernel shape, unsplit, 2 r <= 32
+      const bool fused_gu = !moe && sp.gate_up == 1 && D % 256 == 0 && D < 8192 && F % 64 == 0 &&
+                            (!l.gate_up.lora_a_t || (2 * l.gate_up.rank <= 32 && l.gate_up.r_pad == 32));
       uint16_t* kc = (uint16_t*)s->kv_cache + (size_t)(2 * i) * kv_elems;
       uint16_t* vc = kc + kv_elems;
       TMX_TRY(TMX_K_QKV, qlinear_base(st, w.xn, D, l.qkv.qweight, l.qkv.scales, l.qkv.lora_a_t, nullptr,
@@ -246,6 +249,11 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
         TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
       } else {
+        if (fused_gu) {
+          TMX_TRY(TMX_K_GATE_UP, qlinear_gate_up_swiglu(
+              st, w.xn, D, l.gate_up.qweight, l.gate_up.scales, l.gate_up.lora_a_t, l.gate_up.lora_b,
+              l.gate_up.rank, l.gate_up.lora_scale, w.act, B, D, F, l.gate_up.G));
+        } else {
         const bool gu16 = sp.gate_up == 1;
         TMX_TRY(TMX_K_GATE_UP, qlinear_base(st, w.xn, D, l.gate_up.qweight, l.gate_up.scales,
                                             l.gate_up.lora_a_t, gu16 ? w.y16 : nullptr, w.y_part, w.t_part,
@@ -259,6 +267,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
           a.lora = lora_of(l.gate_up, sp.gate_up);
           a.act = w.act; a.F = F;
           TMX_TRY(TMX_K_SWIGLU, swiglu(st, a, B));
+        }
         }
         TMX_TRY(TMX_K_DOWN, qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t,
                                          nullptr, w.y_part, w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G,

@@ -71,7 +71,10 @@ constexpr int kXStride = kKS * 64 + 8;    // bf16 elements per LDS row
 // LORA = false: one int4 column tile per wave.  LORA = true: the block computes a K-slice
 // of t = x . A from bf16 tiles of A (one 32-column tile per wave); A is stored in MFMA
 // B-fragment order, [K/64][Rpad/32][64 lanes][4 steps][8], so a wave reads 4 KiB contiguously.
-template <int MT, bool LORA>
+// FUSE = true (gate | up pairs with LoRA): every wave also multiplies one of the step's four
+// k-tiles by the 32-column tile of [A_gate | A_up], reusing the activation fragments it already
+// holds, so t = x . A is complete inside the workgroup when the epilogue needs it.
+template <int MT, bool LORA, bool FUSE = false>
 __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)[MT * 32][kXStride]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = lane >> 5, nl = lane & 31;
@@ -101,6 +104,17 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
   for (int m = 0; m < MT; ++m)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
+  // fused LoRA state: accumulators of t, ring of A tiles (this wave's k-tile of each step)
+  f32x16_t tacc[FUSE ? MT : 1];
+  u32x4_t lring[FUSE ? 2 : 1][4];
+  const u32x4_t* lsrc = nullptr;
+  if constexpr (FUSE) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tacc[m][r] = 0.f;
+    lsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + (size_t)lane * 4;  // Rpad == 32: 256 words per k-tile
+  }
 
   // cooperative activation load: chunk c = tid + 256 i -> row c / 32, 16-byte column c % 32
   constexpr int XC = MT * 4;  // chunks per thread and step
@@ -158,6 +172,13 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
 #pragma unroll
     for (int i = 0; i < XC; ++i) *reinterpret_cast<u32x4_t*>(base + xoff_l[i]) = xreg[i];
   };
+  auto load_l = [&](int step, auto dc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value;
+    step = step < last_step ? step : last_step;
+    const size_t kb = (size_t)(kb0 + step * kKS + wave);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) lring[d][t] = lsrc[kb * 256 + t];
+  };
   // one of the four k-tiles of a step
   auto tile_math = [&](int step, int buf, auto dc, auto kc) __attribute__((always_inline)) {
     constexpr int d = decltype(dc)::value, kt = decltype(kc)::value;
@@ -183,6 +204,18 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
       for (int m = 0; m < MT; ++m)
         acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[m], 0, 0, 0);
     }
+    if constexpr (FUSE) {
+      if (wave == kt) {  // this wave's share of t = x . A: k-tile `wave` of every step
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const bf16x8_t b = __builtin_bit_cast(bf16x8_t, lring[d][t]);
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+            tacc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, tacc[m], 0, 0, 0);
+        }
+        load_l(step + DW, dc);
+      }
+    }
   };
   // step s: activations in LDS buffer s & 1, weights in ring slot s % DW
   auto do_step = [&](int step, auto sc) __attribute__((always_inline)) {
@@ -200,6 +233,10 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
   load_x(0);
   load_w(0, IC<0>{});
   if (DW == 2) load_w(1, IC<1 % DW>{});
+  if constexpr (FUSE) {
+    load_l(0, IC<0>{});
+    load_l(1, IC<1>{});
+  }
   stash_x(0);
   __syncthreads();
   const int npairs = nsteps / 2;
@@ -213,6 +250,70 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
     // act = bf16(bf16(g * bf16(sigmoid(g))) * u), g / u = bf16 gate / up projections: the up
     // waves hand their tile to the gate waves through LDS (the slab is free after the last barrier)
     float* ex = reinterpret_cast<float*>(&xs[0][0][0]);  // [2][MT][16][64]
+    // y = bf16(x . W) (+ bf16(bf16(t . B) * ls)): the LoRA product runs on the MFMA, t rows as
+    // A fragments, the B columns of this tile as B fragments, k = rank padded with zeros
+    f32x16_t dl[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dl[m][r] = 0.f;
+    if constexpr (FUSE) {
+      // B fragment of this tile's columns (rows beyond the rank are zero, which also masks
+      // the t columns of the other projection inside the 16-wide k window)
+      bf16x8_t tb;
+      {
+        const int colw = nb * 32 + nl;
+        float bv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int k = h * 8 + j;
+          bv[j] = k < a.lora_r ? bf2f(a.lora_b[(size_t)k * a.N + colw]) : 0.f;
+        }
+        uint32_t pb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pb[j] = pack_bf2(bv[2 * j], bv[2 * j + 1]);
+        __builtin_memcpy(&tb, pb, 16);
+      }
+      // 1. the four waves' partial t tiles meet in LDS   2. summed, rounded to bf16 and laid out
+      // row-major   3. read back as MFMA A fragments
+      float* part = reinterpret_cast<float*>(&xs[0][0][0]);                      // [4][MT][16][64]
+      uint16_t* ts = reinterpret_cast<uint16_t*>(part + 4 * MT * 16 * 64);      // [MT * 32][40]
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part[(((wave * MT + m) * 16 + r) << 6) + lane] = tacc[m][r];
+      __syncthreads();
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int r = wave * 4 + rr;
+          float t = 0.f;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) t += part[(((w * MT + m) * 16 + r) << 6) + lane];
+          ts[(m * 32 + acc_row(r, lane)) * 40 + nl] = f2bf(t);
+        }
+      __syncthreads();
+      const int toff = (wave >= 2) ? a.lora_r : 0;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        uint16_t tv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tv[j] = ts[(m * 32 + nl) * 40 + toff + h * 8 + j];
+        bf16x8_t ta;
+        __builtin_memcpy(&ta, tv, 16);
+        dl[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta, tb, dl[m], 0, 0, 0);
+      }
+      __syncthreads();  // ts / part are overwritten by the exchange below
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float y = rbf(acc[m][r]);
+        if (FUSE) y = rbf(y + rbf(rbf(dl[m][r]) * a.lora_ls));
+        acc[m][r] = y;
+      }
     if (wave >= 2) {
 #pragma unroll
       for (int m = 0; m < MT; ++m)
@@ -228,7 +329,7 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
         for (int r = 0; r < 16; ++r) {
           const int row = m * 32 + acc_row(r, lane);
           if (row >= a.M) continue;
-          const float g = rbf(acc[m][r]), u = rbf(ex[(((wave * MT + m) * 16 + r) << 6) + lane]);
+          const float g = acc[m][r], u = ex[(((wave * MT + m) * 16 + r) << 6) + lane];
           const float sg = rbf(1.f / (1.f + expf(-g)));
           const int drow = a.row_dst ? a.row_dst[row] : row;
           a.y_bf16[(size_t)drow * a.ldy + col] = f2bf(rbf(g * sg) * u);
@@ -258,6 +359,12 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void qlinear_mfma4_kernel(QLi
   __shared__ __align__(16) uint16_t xs[2][MT * 32][kXStride];
   if ((int)blockIdx.x >= a.n_main_blocks) gemm_block4<MT, true>(a, xs);
   else gemm_block4<MT, false>(a, xs);
+}
+
+template <int MT>
+__global__ __launch_bounds__(256, 1) void qlinear_gate_up_kernel(QLinearArgs a) {
+  __shared__ __align__(16) uint16_t xs[2][MT * 32][kXStride];
+  gemm_block4<MT, false, true>(a, xs);
 }
 
 template <int MT>
@@ -620,6 +727,48 @@ int qlinear_num_lora_splits(int K) {
 static int lora_slice_len(int K) {
   const int KT = K / 64, n = qlinear_num_lora_splits(K), g = lora_step(K);
   return ((KT + n - 1) / n + g - 1) / g * g;
+}
+
+// gate | up projection with the LoRA deltas and SwiGLU in the epilogue: act[M, F] =
+// bf16(silu(gate) * up).  Needs the 4-wave kernel (K % 256 == 0, K < 8192) and F % 64 == 0;
+// with LoRA: a_t = [A_gate | A_up] in fragment order with r_pad == 32 (2 r <= 32), lora_b [r][2 F].
+int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
+                           const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
+                           int F, int G) {
+  if (!x || !qw || !scales || !act) return TMX_ERR_ARG;
+  if (M <= 0 || M > 128 || !four_wave(K) || F % 64 || G % 64 || (G & (G - 1)) || K % G || ldx % 8)
+    return TMX_ERR_SHAPE;
+  if (a_t && (!lora_b || r <= 0 || 2 * r > 32)) return TMX_ERR_SHAPE;
+  QLinearArgs a = {};
+  a.fixed_slice = -1;
+  a.x = (const uint16_t*)x;
+  a.ldx = ldx;
+  a.qw = (const uint4*)qw;
+  a.scales = (const uint16_t*)scales;
+  a.a_t = (const uint16_t*)a_t;
+  a.Rpad = 32;
+  a.y_bf16 = (uint16_t*)act;
+  a.ldy = F;
+  a.M = M; a.K = K; a.N = 2 * F; a.G = G;
+  a.nsplit = 1;
+  a.kt_per_split = K / 64;
+  a.pair_off = F / 32;
+  a.lora_b = (const uint16_t*)lora_b;
+  a.lora_r = r;
+  a.lora_ls = ls;
+  a.n_main_blocks = F / 64;
+  auto launch = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3(a.n_main_blocks, 1), dim3(256), 0, st, a);
+    return check_launch();
+  };
+  if (a_t) {
+    if (M <= 32) return launch(qlinear_gate_up_kernel<1>);
+    if (M <= 64) return launch(qlinear_gate_up_kernel<2>);
+    return launch(qlinear_gate_up_kernel<4>);
+  }
+  if (M <= 32) return launch(qlinear_mfma4_kernel<1>);
+  if (M <= 64) return launch(qlinear_mfma4_kernel<2>);
+  return launch(qlinear_mfma4_kernel<4>);
 }
 
 // Host-side dispatch shared by the C entry point and the decode-step launcher.

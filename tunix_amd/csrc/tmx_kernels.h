@@ -23,6 +23,10 @@ struct QLinearArgs {
   const int* row_src;      // activation row of tile row i (null: i)
   const int* row_dst;      // output row of tile row i (null: i)
   int pair_off;            // != 0: gate | up pairing, tile distance between a gate tile and its up tile
+  // LoRA inside the pair epilogue (fused gate | up kernel): a_t = [A_gate | A_up], Rpad == 32
+  const uint16_t* lora_b;  // [lora_r][N] bf16
+  int lora_r;
+  float lora_ls;
 };
 
 // Routed experts (Qwen3 MoE): one launch multiplies, for every expert, the rows routed to it.
@@ -181,6 +185,9 @@ size_t nucleus_bytes(int M, int V);
 size_t head_partial_bytes(int M, int V);
 int qlinear_num_splits(int K, int N, int M);
 int qlinear_num_lora_splits(int K);
+int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
+                           const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
+                           int F, int G);
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
                  int N, int G, int Rpad, int nsplit);
