@@ -256,7 +256,8 @@ def main():
     }
     # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
     mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
-    # projections with K % 256 == 0 below 8192 run the 4-wave kernel, deeper ones the k-way kernel
+    # projections with K % 256 == 0 below 8192 run the 4-wave kernel, deeper ones the k-way
+    # kernel; an unsplit gate|up with LoRA rank <= 16 runs the fused LoRA + SwiGLU kernel
     four = lambda pl: pl.k % 256 == 0 and pl.k < 8192
     dense = [('qkv_linear', 'qkv'), ('o_linear', 'o')]
     symbols = {}
@@ -264,7 +265,14 @@ def main():
       symbols['tmx::moe_expert_kernel<false>'] = ['gate_up_linear']
       symbols['tmx::moe_expert_kernel<true>'] = ['down_linear']
     else:
-      dense += [('gate_up_linear', 'gate_up'), ('down_linear', 'down')]
+      gu = layer0['gate_up']
+      fused = (tot_cnt[CLASS_NAMES.index('swiglu')] == 0 and four(gu))
+      if fused:
+        sym = f'tmx::qlinear_gate_up_kernel<{mt}>' if gu.lora_a_t is not None else f'tmx::qlinear_mfma4_kernel<{mt}>'
+        symbols.setdefault(sym, []).append('gate_up_linear')
+      else:
+        dense.append(('gate_up_linear', 'gate_up'))
+      dense.append(('down_linear', 'down'))
     for cls_name, key in dense:
       sym = f'tmx::qlinear_mfma4_kernel<{mt}>' if four(layer0[key]) else f'tmx::qlinear_mfma_kernel<{mt}, 2>'
       symbols.setdefault(sym, []).append(cls_name)
@@ -287,7 +295,7 @@ def main():
       launches_per_class = {c: int(tot_cnt[idx[c]]) for c in classes}
       byts = float(sum(alg[c] * launches_per_class[c] for c in classes)) / n
       avg = t / n
-      per_symbol[sym] = {'total_ms_per_step': avg * n / max(ctx_n, 1), 'launches_per_step': n / max(ctx_n, 1),
+      per_symbol[sym] = {'classes': classes, 'total_ms_per_step': avg * n / max(ctx_n, 1), 'launches_per_step': n / max(ctx_n, 1),
                          'avg_launch_ms': avg,
                          'algorithmic_bytes_per_launch': byts,
                          'achieved_GBps': byts / (avg * 1e-3) / 1e9, 'frac': byts / (avg * 1e-3) / 8e12}
@@ -304,7 +312,7 @@ def main():
                           'algorithmic_bytes_per_launch': d['algorithmic_bytes_per_launch'],
                           'note': 'mean HIP-event time around the launches of this kernel in the sampled '
                                   'steps (includes event packet processing, see empty_launch_event_pair_ms); '
-                                  'the 4-wave projection kernel serves qkv, o and gate|up, the k-way kernel down'}
+                                  'classes per kernel symbol are listed in roofline_kernels'}
     result['roofline_kernels'] = per_symbol
     result['roofline_all'] = {}
     for i, n in enumerate(CLASS_NAMES):
