@@ -109,6 +109,7 @@ def main():
   ap.add_argument('--workload', default='llama3.1-8b-grpo', choices=sorted(WORKLOADS))
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--no-profile', action='store_true')
+  ap.add_argument('--graph', action='store_true', help='replay one recorded decode step (tmx_decode_steps_graph)')
   ap.add_argument('--sync-steps', action='store_true',
                   help='synchronise after every decode step (counter-collection runs: the profiler '
                        'cannot hold tens of thousands of pending dispatches)')
@@ -163,7 +164,7 @@ def main():
 
   def run(st, n, sample=True):
     if not args.sync_steps:
-      return sampler.run_steps(st, n, sample=sample)
+      return sampler.run_steps(st, n, sample=sample, graph=args.graph)
     for _ in range(n):
       sampler.run_steps(st, 1, sample=sample)
       torch.cuda.synchronize()

@@ -256,6 +256,14 @@ size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int ca
 int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
                      int n_steps, int sample);
 
+/* The same steps with one of them recorded into a HIP graph and replayed n_steps - 1 times
+ * (fewer host launches; what the reference gets from jit-compiling the while_loop).  Unlike
+ * tmx_decode_steps this call WAITS for its replays before it returns (the graph is private
+ * to the call), creates and destroys a stream, an event and a graph, and falls back to plain
+ * launches for the sorting branch of top-p, for n_steps < 4 or when capture is unavailable. */
+int tmx_decode_steps_graph(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
+                           int n_steps, int sample);
+
 /* Measurement aid (no counterpart in the reference): the same as tmx_decode_steps, but every
  * kernel launch is bracketed by HIP events on `stream`; after enqueuing, the call SYNCHRONISES
  * the stream and adds up the elapsed milliseconds and the launch count per kernel class into

@@ -288,3 +288,34 @@ def test_moe_decoder_matches_oracle():
   # logits of this model reach |z| in [1, 2): one bf16 ulp of the chosen token's logit (2^-7, from
   # another f32 summation order) moves its logprob by as much, on top of the 1e-2 budget
   _compare_greedy(out, ref, 4, min_checked=20, lp_extra=2.0 ** -7)
+
+
+def test_graph_replay_matches_plain_launches_on_every_replay():
+  """tmx_decode_steps_graph against tmx_decode_steps: several graph calls in a row, with the
+  program's own eager work (a plain step, host reads) and synchronisation between them; every
+  call's tokens, logprobs, KV cache and step counter equal the plain launches'."""
+  cfg = C.TOY
+  _, model = _pair(cfg, seed=17, targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
+  rng = np.random.default_rng(2)
+  ids = np.stack([rng.integers(3, cfg.vocab_size, 8) for _ in range(4)]).astype(np.int32)
+  def run(graph):
+    s = _sampler(model, cfg, 64)
+    s.eos_ids = np.array([-1])
+    st = s.init_sample_state(ids, 64, False, None, 0.9, 1.0, None, 5, include_logprobs=True,
+                             prompt_lengths=np.full(4, 8))
+    snaps = []
+    s.run_steps(st, 7, sample=False, graph=graph)
+    for n in (9, 1, 12, 5, 16):
+      s.run_steps(st, n, sample=True, graph=graph)
+      torch.cuda.synchronize()
+      snaps.append((st['token_buffer'].cpu().numpy().copy(), st['logprobs'].cpu().numpy().copy(),
+                    int(st['step'].item()), st['cache'].float().abs().sum().item()))
+      s.run_steps(st, 1, sample=True, graph=False)   # eager work between the replays
+      _ = st['done'].cpu()
+    return snaps
+  plain, replay = run(False), run(True)
+  for (t0, l0, s0, c0), (t1, l1, s1, c1) in zip(plain, replay):
+    assert s0 == s1
+    np.testing.assert_array_equal(t0, t1)
+    np.testing.assert_array_equal(l0, l1)
+    assert c0 == c1

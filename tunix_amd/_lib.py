@@ -33,6 +33,7 @@ SIGNATURES = {
     'tmx_moe_route': [vp, vp, vp, ci, ci, ci, ci, vp, vp],
     'tmx_moe_experts': [vp, vp, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, vp, ci],
     'tmx_decode_steps': [vp, vp, vp, ci, ci],
+    'tmx_decode_steps_graph': [vp, vp, vp, ci, ci],
     'tmx_decode_steps_profiled': [vp, vp, vp, ci, ci, vp, vp],
 }
 # entry points that return size_t

@@ -323,6 +323,53 @@ extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state*
   return decode_steps_impl(m, s, stream, n_steps, sample, nullptr);
 }
 
+// One decode step recorded into a HIP graph and replayed: the step index lives on the device,
+// so every replay is the same list of launches.  The first step runs eagerly (it also performs
+// the one-time kernel attribute set-up), the capture happens on a private stream that is ordered
+// after `stream` by events, and the replays are launched back on `stream`.
+extern "C" int tmx_decode_steps_graph(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
+                                      int n_steps, int sample) {
+  if (n_steps < 4 || !m || !s) return decode_steps_impl(m, s, stream, n_steps, sample, nullptr);
+  // the sorting branch of top-p calls a library sort that records memset nodes: keep it eager
+  if (sample && s->sampling_mode == TMX_SAMPLE_TOP_P && (s->top_p < 1.0f || s->top_k > 0))
+    return decode_steps_impl(m, s, stream, n_steps, sample, nullptr);
+  int rc = decode_steps_impl(m, s, stream, 1, sample, nullptr);
+  if (rc != TMX_OK) return rc;
+  hipStream_t user = (hipStream_t)stream;
+  hipStream_t cap = nullptr;
+  hipEvent_t ev = nullptr;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  rc = TMX_ERR_LAUNCH;
+  bool captured = false;
+  do {
+    if (hipStreamCreateWithFlags(&cap, hipStreamNonBlocking) != hipSuccess) break;
+    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) break;
+    if (hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal) != hipSuccess) break;
+    const int crc = decode_steps_impl(m, s, cap, 1, sample, nullptr);
+    const hipError_t e = hipStreamEndCapture(cap, &graph);
+    if (crc != TMX_OK) { rc = crc; break; }
+    if (e != hipSuccess || !graph) break;
+    if (hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess) break;
+    captured = true;
+    rc = TMX_OK;
+    for (int i = 1; i < n_steps; ++i)
+      if (hipGraphLaunch(exec, user) != hipSuccess) { rc = TMX_ERR_LAUNCH; break; }
+    // the graph objects may only go once the replays have run
+    if (hipEventRecord(ev, user) == hipSuccess) (void)hipEventSynchronize(ev);
+    else (void)hipStreamSynchronize(user);
+  } while (false);
+  if (exec) (void)hipGraphExecDestroy(exec);
+  if (graph) (void)hipGraphDestroy(graph);
+  if (ev) (void)hipEventDestroy(ev);
+  if (cap) (void)hipStreamDestroy(cap);
+  if (!captured && rc == TMX_ERR_LAUNCH) {
+    (void)hipGetLastError();
+    return decode_steps_impl(m, s, stream, n_steps - 1, sample, nullptr);  // capture unavailable
+  }
+  return rc;
+}
+
 extern "C" int tmx_decode_steps_profiled(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
                                          int n_steps, int sample, float* class_ms_host,
                                          int* class_launches_host) {

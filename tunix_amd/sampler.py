@@ -89,6 +89,9 @@ class Sampler:
     self._cache = None
     self._workspace = None
     self._nucleus_ws = None
+    # replay one recorded decode step instead of launching every kernel: measured neutral on
+    # MI355X (the steps are bound by the device, not by host launches), so off by default
+    self.use_graph = False
     self.eos_ids = None
     self.last_step_logits = None
 
@@ -217,14 +220,16 @@ class Sampler:
       s.nucleus_workspace, s.nucleus_workspace_bytes = self._nucleus_ws.data_ptr(), self._nucleus_ws.numel()
     return s
 
-  def run_steps(self, st, n_steps, sample=True):
-    """Enqueues n decode-loop iterations on the current stream (no host sync)."""
+  def run_steps(self, st, n_steps, sample=True, graph=False):
+    """Runs n decode-loop iterations on the current stream.  graph=False only enqueues (no host
+    sync); graph=True replays one recorded step and returns when the steps have run."""
     if n_steps <= 0:
       return
     cs = self._c_state(st)
-    rc = self._lib.tmx_decode_steps(ctypes.byref(self._transformer.desc()), ctypes.byref(cs),
-                                    _lib.stream(), int(n_steps), 1 if sample else 0)
-    _lib.check(rc, 'tmx_decode_steps')
+    fn = self._lib.tmx_decode_steps_graph if graph else self._lib.tmx_decode_steps
+    rc = fn(ctypes.byref(self._transformer.desc()), ctypes.byref(cs), _lib.stream(), int(n_steps),
+            1 if sample else 0)
+    _lib.check(rc, 'tmx_decode_steps_graph' if graph else 'tmx_decode_steps')
 
   # -- the call ---------------------------------------------------------------
   def __call__(self, input_strings=None, max_generation_steps=0, max_prompt_length=None, echo=False,
@@ -259,11 +264,11 @@ class Sampler:
     logits_steps = []
     if max_generation_steps > 0:
       # cache fill over prompt columns 0 .. P-2, then P-1 produces generated token #1
-      self.run_steps(st, p - 1, sample=False)
+      self.run_steps(st, p - 1, sample=False, graph=self.use_graph)
       remaining = max_generation_steps
       while remaining > 0:
         n = 1 if return_logits else min(self.CHECK_EVERY, remaining)
-        self.run_steps(st, n, sample=True)
+        self.run_steps(st, n, sample=True, graph=self.use_graph)
         remaining -= n
         if return_logits:
           logits_steps.append(st['logits'].clone())
