@@ -255,6 +255,8 @@ def main():
         'attention': batch * ctx * cfg.num_kv_heads * cfg.head_dim * 2 * 2,
         'head_sample': hbytes,
     }
+    if not cfg.num_experts and tot_cnt[CLASS_NAMES.index('swiglu')] == 0:
+      alg['gate_up_linear'] -= batch * cfg.hidden_dim * 2  # fused SwiGLU: [M, F] goes out, not [M, 2 F]
     # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
     mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
     # projections with K % 256 == 0 below 8192 run the 4-wave kernel, deeper ones the k-way
