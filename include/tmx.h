@@ -48,6 +48,9 @@ extern "C" {
 
 #define TMX_SAMPLE_GREEDY 0
 #define TMX_SAMPLE_TOP_P 1
+#define TMX_SAMPLE_SCORE 2 /* teacher forcing: no token is chosen; logprobs[m, *step + 1] =
+                              log_softmax(logits / temperature)[token_buffer[m, *step + 1]]
+                              (tunix/rl/common.py:426-606 compute_per_token_logps) */
 
 const char* tmx_status_string(int status);
 int tmx_abi_version(void);

@@ -260,8 +260,6 @@ def test_lora_update_params_and_rollout_surface():
                                       eos_tokens=[-1], return_logprobs=True, seed=3), prompt_token_ids=prompts)
   assert len(ro.tokens) == 2 and all(len(t) == 5 for t in ro.tokens) and len(ro.logprobs[0]) == 5
   assert ro.left_padded_prompt_tokens.shape == (2, 8)
-  with pytest.raises(NotImplementedError):
-    r.get_per_token_logps(None, None)
 
 
 def test_unsupported_sampling_modes_fail_loudly():
@@ -319,3 +317,40 @@ def test_graph_replay_matches_plain_launches_on_every_replay():
     np.testing.assert_array_equal(t0, t1)
     np.testing.assert_array_equal(l0, l1)
     assert c0 == c1
+
+
+def test_per_token_logps_match_oracle_and_the_rollout_logprobs():
+  """Scoring pass of the rollout adapter (tunix/rl/common.py:426-606): left-padded prompts,
+  right-padded completions; against the oracle's full-sequence forward, and against the
+  log-probs the Sampler itself reported when it generated the same tokens at T = 1."""
+  from oracle import scoring
+  cfg = C.TOY
+  oracle, model = _pair(cfg, seed=23)
+  s = _sampler(model, cfg, 48)
+  rng = np.random.default_rng(9)
+  pad = 0
+  prompt = np.full((4, 10), pad, np.int32)
+  comp = np.full((4, 12), pad, np.int32)
+  for b, (pl, cl) in enumerate(((10, 12), (7, 9), (3, 12), (10, 1))):
+    prompt[b, 10 - pl:] = rng.integers(3, cfg.vocab_size, pl)
+    comp[b, :cl] = rng.integers(3, cfg.vocab_size, cl)
+  got = s.per_token_logps(prompt, comp, pad_id=pad)
+  want = scoring.per_token_logps(oracle, prompt, comp, pad)
+  valid = comp != pad
+  assert got.shape == (4, 12)
+  assert np.abs(got - want)[valid].max() <= LOGPROB_TOL, np.abs(got - want)[valid].max()
+  # temperature scaling
+  got_t = s.per_token_logps(prompt, comp, pad_id=pad, temperature=0.7)
+  want_t = scoring.per_token_logps(oracle, prompt, comp, pad, temperature=0.7)
+  assert np.abs(got_t - want_t)[valid].max() <= 2 * LOGPROB_TOL
+  # the rollout's own log-probs: generate at T = 1, then score the generated tokens
+  r = TmxRollout(rollout_actor=model, tokenizer=C.ToyTokenizer(), mesh=None,
+                 rollout_config=RolloutConfig(kv_cache_size=48))
+  prompts = [prompt[b, prompt[b] != pad] for b in range(4)]
+  ro = r.generate(None, RolloutConfig(max_tokens_to_generate=8, max_prompt_length=10, temperature=1.0, top_p=1.0,
+                                      eos_tokens=[-1], return_logprobs=True, seed=3), prompt_token_ids=prompts)
+  gen = np.stack(ro.tokens)
+  scored = r.get_per_token_logps(ro.left_padded_prompt_tokens, gen)
+  np.testing.assert_allclose(scored, np.stack(ro.logprobs), atol=2e-5)
+  with pytest.raises(ValueError):
+    s.per_token_logps(np.zeros((2, 0), np.int32), comp[:2])

@@ -128,7 +128,14 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
   // per-step key = fold_in(seed, step)
   uint32_t key0 = 0, key1 = 0;
   if (a.mode == TMX_SAMPLE_TOP_P) threefry2x32(a.k0, a.k1, 0u, (uint32_t)*a.step, key0, key1);
+  const bool score = a.mode == TMX_SAMPLE_SCORE;
 
+  int target[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int row = m * 32 + nl;
+    target[m] = (score && row < a.M) ? a.token_buffer[(size_t)row * a.buf_len + *a.step + 1] : -1;
+  }
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     const int row = m * 32 + nl;
@@ -143,7 +150,11 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
         for (int f = 0; f < a.n_forbidden; ++f)
           if (a.forbidden[f] == v) logit = -INFINITY;
         float z = logit, key = logit;
-        if (a.mode == TMX_SAMPLE_TOP_P) {
+        if (score) {
+          // the "best" candidate is the given next token: its z is what the log-prob needs
+          z = logit / a.temperature;
+          key = (v == target[m]) ? 0.f : -INFINITY;
+        } else if (a.mode == TMX_SAMPLE_TOP_P) {
           z = logit / a.temperature;
           if (a.sort_keys) {
             // ascending key order = descending z (with -0 == +0), rows kept apart by the high word
@@ -235,6 +246,10 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
       best_merge(best, o);
     }
     const int col = *a.step + 1;
+    if (a.mode == TMX_SAMPLE_SCORE) {  // teacher forcing: the token stays, only its log-prob is written
+      if (a.logprobs) a.logprobs[(size_t)row * a.buf_len + col] = (best.z - mx) - logf(se);
+      return;
+    }
     const int tok = best.idx;
     a.token_buffer[(size_t)row * a.buf_len + col] = tok;
     if (a.logprobs) a.logprobs[(size_t)row * a.buf_len + col] = (best.z - mx) - logf(se);
@@ -278,7 +293,7 @@ extern "C" int tmx_head_sample(void* stream, const void* x, const void* head_w, 
                                uint8_t* done, int buf_len, float* logits_out, void* workspace) {
   if (!x || !head_w || !step || !token_buffer || !done || !workspace) return TMX_ERR_ARG;
   if ((n_forbidden > 0 && !forbidden) || (n_eos > 0 && !eos)) return TMX_ERR_ARG;
-  if (mode != TMX_SAMPLE_GREEDY && mode != TMX_SAMPLE_TOP_P) return TMX_ERR_UNSUPPORTED;
+  if (mode != TMX_SAMPLE_GREEDY && mode != TMX_SAMPLE_TOP_P && mode != TMX_SAMPLE_SCORE) return TMX_ERR_UNSUPPORTED;
   HeadArgs a = {};
   a.x = (const uint16_t*)x;
   a.w = (const uint16_t*)head_w;

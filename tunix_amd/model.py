@@ -15,7 +15,7 @@ from tunix_amd import quant
 from tunix_amd import _lib
 
 FAMILY_LLAMA3, FAMILY_QWEN3 = 0, 1
-SAMPLE_GREEDY, SAMPLE_TOP_P = 0, 1
+SAMPLE_GREEDY, SAMPLE_TOP_P, SAMPLE_SCORE = 0, 1, 2
 MAX_RPAD = 128
 
 

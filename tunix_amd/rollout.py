@@ -81,8 +81,8 @@ class TmxRollout(BaseRollout):
         prompt_lengths=out.prompt_lengths)
 
   def get_per_token_logps(self, prompt_tokens, completion_tokens):
-    raise NotImplementedError(
-        'the teacher-forced scoring pass (tunix/rl/common.py:426-606) is not part of the decode path')
+    """vanilla_rollout.py:75-88: compute_per_token_logps with this rollout's pad id."""
+    return self._sampler.per_token_logps(prompt_tokens, completion_tokens, pad_id=self.pad_id())
 
   def update_params(self, params, filter_types=None):
     self._sampler.update_params(params, filter_types)

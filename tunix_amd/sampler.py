@@ -16,7 +16,7 @@ import torch
 from tunix_amd import _lib
 from tunix_amd import utils
 from tunix_amd.configs import CacheConfig, SamplerOutput
-from tunix_amd.model import DecodeState, SAMPLE_GREEDY, SAMPLE_TOP_P
+from tunix_amd.model import DecodeState, SAMPLE_GREEDY, SAMPLE_TOP_P, SAMPLE_SCORE
 
 _REQUIRED_TOKENIZER_METHODS = ('encode', 'decode', 'bos_id', 'eos_id', 'pad_id')
 
@@ -200,7 +200,7 @@ class Sampler:
     s.input_mask, s.done, s.step = st['input_mask'].data_ptr(), st['done'].data_ptr(), st['step'].data_ptr()
     s.logprobs = st['logprobs'].data_ptr() if st['logprobs'] is not None else None
     s.kv_cache = st['cache'].data_ptr()
-    s.sampling_mode = SAMPLE_GREEDY if st['sampling_mode'] == 'greedy' else SAMPLE_TOP_P
+    s.sampling_mode = {'greedy': SAMPLE_GREEDY, 'top_p': SAMPLE_TOP_P, 'score': SAMPLE_SCORE}[st['sampling_mode']]
     s.temperature = st['temperature']
     s.top_p = 1.0 if st['top_p'] is None else float(st['top_p'])
     s.top_k = int(st['top_k']) if st['top_k'] else 0
@@ -230,6 +230,43 @@ class Sampler:
     rc = fn(ctypes.byref(self._transformer.desc()), ctypes.byref(cs), _lib.stream(), int(n_steps),
             1 if sample else 0)
     _lib.check(rc, 'tmx_decode_steps_graph' if graph else 'tmx_decode_steps')
+
+  def per_token_logps(self, prompt_tokens, completion_tokens, pad_id=None, temperature=1.0, token_mask=None):
+    """Teacher-forced log-probabilities of the completion tokens, f32 [B, completion_len]:
+    log_softmax(logits / temperature)[token] at every completion position given everything
+    before it (tunix/rl/common.py:426-606 compute_per_token_logps without sequence packing;
+    positions and the attention mask follow process_ids, :257-330: valid = token != pad_id or
+    `token_mask`).  Entries at padded completion positions are computed like the reference's
+    and meant to be masked by the caller.  The sequence is walked token by token through the
+    decode kernels."""
+    prompt = np.asarray(prompt_tokens, dtype=np.int32)
+    comp = np.asarray(completion_tokens, dtype=np.int32)
+    if prompt.ndim != 2 or comp.ndim != 2 or prompt.shape[0] != comp.shape[0]:
+      raise ValueError('prompt_tokens and completion_tokens must be [B, P] and [B, T]')
+    pad = self.tokenizer.pad_id() if pad_id is None else pad_id
+    ids = np.concatenate([prompt, comp], axis=1)
+    b, total = ids.shape
+    p, t = prompt.shape[1], comp.shape[1]
+    if total > self.cache_config.cache_size:
+      raise ValueError(f'Total sampling steps {total} must be less than the cache size'
+                       f' {self.cache_config.cache_size}.')
+    if p == 0:
+      raise ValueError('prompt_tokens must hold at least one column (packed sequences are not supported)')
+    if t == 0:
+      return np.zeros((b, 0), np.float32)
+    valid = (ids != pad) if token_mask is None else np.asarray(token_mask).astype(bool)
+    if valid.shape != ids.shape:
+      raise ValueError('token_mask must match the full prompt/completion shape')
+    self.eos_ids = np.array([-1])
+    st = self.init_sample_state(ids, total, False, None, temperature if temperature not in (0.0, 1.0) else 1.0,
+                                1.0, None, 0, include_logprobs=True)
+    dev = self._transformer.device
+    st['input_mask'] = torch.from_numpy(valid.astype(np.uint8)).to(dev)
+    st['positions'] = torch.from_numpy(utils.build_positions_from_mask(valid).astype(np.int32)).to(dev)
+    st['sampling_mode'] = 'score'
+    self.run_steps(st, p - 1, sample=False)
+    self.run_steps(st, t, sample=True)
+    return st['logprobs'][:, p:p + t].cpu().numpy()
 
   # -- the call ---------------------------------------------------------------
   def __call__(self, input_strings=None, max_generation_steps=0, max_prompt_length=None, echo=False,
