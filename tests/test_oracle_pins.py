@@ -364,3 +364,29 @@ def test_oracle_sampler_loop_invariants():
   assert not (set(np.concatenate(fb['tokens']).tolist()) & set(banned))
   with pytest.raises(ValueError, match='must be less than the cache size'):
     OSAM.generate(dec, cfg, prompts, 20, 16, max_prompt_length=8)
+
+
+def test_scoring_pass_reproduces_the_logprobs_of_generation():
+  """oracle.scoring (full-sequence forward, no cache) against the sampler loop (prefill + cached
+  decode): scoring the tokens a greedy rollout produced returns the log-probs it reported, and
+  a hand-built 2-row case checks the gather / slicing convention of compute_per_token_logps
+  (logit at position i scores token i + 1; completion slice only)."""
+  from oracle import sampler as OSAM
+  from oracle import scoring
+  cfg = OM.Config('llama3', 2, 64, 64, 128, 2, 32, 2, rope_theta=10000, norm_eps=1e-5, tied=True)
+  dec = OM.Decoder(cfg, OM.random_weights(cfg, 3, 64, 4, 8.0, ('q', 'v')))
+  rng = np.random.default_rng(1)
+  prompts = [rng.integers(3, 64, n) for n in (5, 3)]
+  ref = OSAM.generate(dec, cfg, prompts, 6, 16, eos_ids=(-1,))
+  comp = np.stack(ref['tokens'])
+  got = scoring.per_token_logps(dec, ref['padded_prompt_tokens'], comp, 0)
+  np.testing.assert_allclose(got, np.stack(ref['logprobs']), atol=2e-3)
+  # slicing convention, by hand: one forward over the concatenation
+  ids = np.concatenate([ref['padded_prompt_tokens'], comp], axis=1)
+  valid = ids != 0
+  logits, _ = dec(ids, OMK.build_positions_from_mask(valid), None, OMK.make_causal_attn_mask(valid, ids.shape[1]))
+  lp = OS.log_softmax(logits)
+  p = ref['padded_prompt_tokens'].shape[1]
+  for b in range(2):
+    for t in range(comp.shape[1]):
+      assert got[b, t] == lp[b, p + t - 1, comp[b, t]]
