@@ -49,7 +49,7 @@ def _compare_greedy(out, ref, n_rows, min_checked, lp_extra=0.0):
 
 
 def test_toy_config_greedy_matches_oracle():
-  """BASELINE config 1: 2 layers, d 256, 4 heads, SwiGLU 1024, vocab 1024, int4 g64, LoRA r8 on
+  """The toy configuration of the benchmark description: 2 layers, d 256, 4 heads, SwiGLU 1024, vocab 1024, int4 g64, LoRA r8 on
   q/k/v/o, batch 4 x 32 prompt tokens, 32 greedy steps."""
   cfg = C.TOY
   oracle, model = _pair(cfg)

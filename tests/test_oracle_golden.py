@@ -1,7 +1,11 @@
 """The oracle against every golden vector the reference's own tests hold for this path
 (tests/generate/utils_test.py:91-179, tests/generate/sampler_test.py:1095-1132) and the
-Random123 known-answer vectors for threefry2x32.  The product's host helpers
+Random123 known-answer vectors for threefry2x32, all kept as data in
+tests/golden/reference_vectors.json.  The product's host helpers
 (tunix_amd.utils) are checked against the same vectors."""
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -10,62 +14,58 @@ from oracle import prng
 from tunix_amd import utils as PU
 
 IMPLS = [pytest.param(OM, id='oracle'), pytest.param(PU, id='product')]
+GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'reference_vectors.json')))
 
 
 @pytest.mark.parametrize('m', IMPLS)
 def test_compute_attention_mask_golden(m):
-  # tests/generate/utils_test.py:91-113
-  input_mask = np.array([[1, 1, 0, 0, 0], [1, 1, 0, 1, 0]], dtype=bool)
-  got = m.compute_attention_masks(4, 8, input_mask)
-  want = np.array([[0, 0, 1, 1, 1, 0, 0, 0], [0, 0, 1, 0, 1, 0, 0, 0]], dtype=bool)
-  assert got.shape == (2, 1, 8)
-  np.testing.assert_array_equal(got[:, 0], want)
-  # ring case: total sampling steps longer than the cache
-  got = m.compute_attention_masks(4, 4, input_mask)
-  want = np.array([[0, 1, 1, 1], [0, 1, 0, 1]], dtype=bool)
-  np.testing.assert_array_equal(got[:, 0], want)
+  g = GOLD['compute_attention_masks']
+  input_mask = np.array(g['input_mask'], dtype=bool)
+  for case in g['cases']:
+    got = m.compute_attention_masks(case['time_step'], case['seq_len'], input_mask)
+    assert got.shape == (2, 1, case['seq_len'])
+    np.testing.assert_array_equal(got[:, 0], np.array(case['expected'], dtype=bool))
 
 
 @pytest.mark.parametrize('m', IMPLS)
 def test_make_causal_attn_mask_golden(m):
-  # tests/generate/utils_test.py:115-132
-  got = m.make_causal_attn_mask(np.array([[0, 1, 1, 0], [1, 1, 1, 0]]), 5)
-  want = np.array([
-      [[0, 0, 0, 0, 0], [0, 1, 0, 0, 0], [0, 1, 1, 0, 0], [0, 1, 1, 0, 0]],
-      [[1, 0, 0, 0, 0], [1, 1, 0, 0, 0], [1, 1, 1, 0, 0], [1, 1, 1, 0, 0]],
-  ])
-  np.testing.assert_array_equal(got.astype(int), want)
+  g = GOLD['make_causal_attn_mask']
+  got = m.make_causal_attn_mask(np.array(g['input_mask']), g['cache_size'])
+  np.testing.assert_array_equal(got.astype(int), np.array(g['expected']))
 
 
 @pytest.mark.parametrize('m', IMPLS)
 def test_next_power_of_2_and_cdiv_golden(m):
-  # tests/generate/utils_test.py:134-150
-  assert [m.next_power_of_2(x) for x in (0, 2, 3, 4, 5)] == [1, 2, 4, 4, 8]
-  for a, b, want in ((0, 4, 0), (1, 4, 1), (4, 4, 1), (5, 4, 2), (8, 4, 2), (7, 1, 7)):
+  g = GOLD['next_power_of_2']
+  assert [m.next_power_of_2(x) for x in g['inputs']] == g['expected']
+  for a, b, want in GOLD['cdiv']['cases']:
     assert m.cdiv(a, b) == want
 
 
 @pytest.mark.parametrize('m', IMPLS)
 def test_index_finders_golden(m):
-  # tests/generate/utils_test.py:152-179
-  for ids, want in (([1, 2, 3, 4, 5, 6], 0), ([0, 0, 1, 2, 3, 4], 2), ([0, 1, 2, 3, 0, 0], 1)):
-    assert m.find_first_non_pad_idx(np.array(ids), 0) == want
-  for ids, want in (([1, 2, 3, 4, 5, -1], 5), ([1, 2, -1, 4, -1, 0], 2), ([1, 2, 3, 4, 5, 6], 6)):
-    assert m.find_first_eos_idx(np.array(ids), -1) == want
-  for ids, want in (([1, 2, 3, 4, 5, 6], 5), ([1, 2, 3, 0, 0, 0], 2), ([0, 1, 2, 3, 0, 0], 3)):
-    assert m.find_last_non_pad_idx(np.array(ids), 0) == want
+  g = GOLD['find_first_non_pad_idx']
+  for ids, want in g['cases']:
+    assert m.find_first_non_pad_idx(np.array(ids), g['pad_id']) == want
+  g = GOLD['find_first_eos_idx']
+  for ids, want in g['cases']:
+    assert m.find_first_eos_idx(np.array(ids), g['eos_id']) == want
+  g = GOLD['find_last_non_pad_idx']
+  for ids, want in g['cases']:
+    assert m.find_last_non_pad_idx(np.array(ids), g['pad_id']) == want
 
 
 @pytest.mark.parametrize('m', IMPLS)
 def test_left_pad_and_positions_golden(m):
-  # tests/generate/sampler_test.py:1078-1132: prompt_token_ids [[0, 3], [4, 0, 5]] at P = 4
-  ids, lens, p = m.left_pad_prompt_tokens([[0, 3], [4, 0, 5]], 4, 0, max_allowed_length=14)
-  np.testing.assert_array_equal(ids, np.array([[0, 0, 0, 3], [0, 4, 0, 5]], np.int32))
-  np.testing.assert_array_equal(lens, np.array([2, 3], np.int32))
-  assert p == 4
-  mask = np.arange(4)[None, :] >= (4 - lens[:, None])
-  np.testing.assert_array_equal(mask, [[False, False, True, True], [False, True, True, True]])
-  np.testing.assert_array_equal(m.build_positions_from_mask(mask), [[0, 0, 0, 1], [0, 0, 1, 2]])
+  g = GOLD['left_pad_and_positions']
+  ids, lens, p = m.left_pad_prompt_tokens(g['prompt_token_ids'], g['max_prompt_length'], g['pad_id'],
+                                          max_allowed_length=14)
+  np.testing.assert_array_equal(ids, np.array(g['padded_prompt_tokens'], np.int32))
+  np.testing.assert_array_equal(lens, np.array(g['prompt_lengths'], np.int32))
+  assert p == g['max_prompt_length']
+  mask = np.arange(p)[None, :] >= (p - lens[:, None])
+  np.testing.assert_array_equal(mask, np.array(g['input_mask'], dtype=bool))
+  np.testing.assert_array_equal(m.build_positions_from_mask(mask), g['positions'])
 
 
 @pytest.mark.parametrize('m', IMPLS)
@@ -80,13 +80,12 @@ def test_left_pad_bucketing(m):
 
 
 def test_threefry2x32_known_answers():
-  # Random123 kat_vectors, threefry2x32 with 20 rounds
-  def run(k0, k1, c0, c1):
-    x0, x1 = prng.threefry2x32(np.uint32(k0), np.uint32(k1), np.uint32(c0), np.uint32(c1))
-    return int(x0), int(x1)
-  assert run(0, 0, 0, 0) == (0x6B200159, 0x99BA4EFE)
-  assert run(0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF) == (0x1CB996FC, 0xBB002BE7)
-  assert run(0x13198A2E, 0x03707344, 0x243F6A88, 0x85A308D3) == (0xC4923A9C, 0x483DF7A0)
+  num = lambda v: int(v, 16) if isinstance(v, str) else int(v)
+  for case in GOLD['threefry2x32']['cases']:
+    k0, k1 = (np.uint32(num(v)) for v in case['key'])
+    c0, c1 = (np.uint32(num(v)) for v in case['counter'])
+    x0, x1 = prng.threefry2x32(k0, k1, c0, c1)
+    assert (int(x0), int(x1)) == tuple(num(v) for v in case['expected'])
 
 
 def test_uniform_and_gumbel_ranges():
