@@ -259,9 +259,9 @@ def main():
       alg['gate_up_linear'] -= batch * cfg.hidden_dim * 2  # fused SwiGLU: [M, F] goes out, not [M, 2 F]
     # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
     mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
-    # projections with K % 256 == 0 below 8192 run the 4-wave kernel, deeper ones the k-way
-    # kernel; an unsplit gate|up with LoRA rank <= 16 runs the fused LoRA + SwiGLU kernel
-    four = lambda pl: pl.k % 256 == 0 and pl.k < 8192
+    # projections with K % 256 == 0 below 8192 run the 4-wave kernel, deeper or mid-width ones (40
+    # to 191 column blocks) the k-way kernel; an unsplit gate|up with LoRA rank <= 16 runs the fused LoRA + SwiGLU kernel
+    four = lambda pl: pl.k % 256 == 0 and pl.k < 8192 and not (40 <= (pl.n + 127) // 128 < 192)
     dense = [('qkv_linear', 'qkv'), ('o_linear', 'o')]
     symbols = {}
     if cfg.num_experts:
@@ -269,7 +269,7 @@ def main():
       symbols['tmx::moe_expert_kernel<true>'] = ['down_linear']
     else:
       gu = layer0['gate_up']
-      fused = (tot_cnt[CLASS_NAMES.index('swiglu')] == 0 and four(gu))
+      fused = (tot_cnt[CLASS_NAMES.index('swiglu')] == 0 and gu.k % 256 == 0 and gu.k < 8192)
       if fused:
         sym = f'tmx::qlinear_gate_up_kernel<{mt}>' if gu.lora_a_t is not None else f'tmx::qlinear_mfma4_kernel<{mt}>'
         symbols.setdefault(sym, []).append('gate_up_linear')

@@ -77,11 +77,11 @@ int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const voi
 
 /* The matrix product alone, for callers that fuse their own consumer: writes `nsplit` f32
  * K-slice planes y_part[nsplit][M][N] (their sum is x . dequant(W)) and, with LoRA,
- * t_part[tmx_qlora_linear_num_lora_splits(K)][M][TMX_MAX_RPAD] (their sum is x . A).
+ * t_part[tmx_qlora_linear_num_lora_splits(K, N)][M][TMX_MAX_RPAD] (their sum is x . A).
  * nsplit in [1, TMX_MAX_SPLITS] and such that no K-slice is empty;
  * tmx_qlora_linear_num_splits() returns the count the library itself would pick. */
 int tmx_qlora_linear_num_splits(int M, int K, int N);
-int tmx_qlora_linear_num_lora_splits(int K);
+int tmx_qlora_linear_num_lora_splits(int K, int N);
 int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight, const void* scales,
                             const void* lora_a_t, float* y_part, float* t_part, int M, int K, int N,
                             int G, int r_pad, int nsplit);

@@ -148,7 +148,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     if (l.lora_a_t) {
       li.t_part = w.t_part;
       li.ldt = TMX_MAX_RPAD;
-      li.nsplit = qlinear_num_lora_splits(l.K);
+      li.nsplit = qlinear_num_lora_splits(l.K, l.N);
       li.b = (const uint16_t*)l.lora_b;
       li.r = l.rank;
       li.ls = l.lora_scale;

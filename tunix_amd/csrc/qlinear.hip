@@ -671,7 +671,14 @@ static int launch_qlinear(hipStream_t st, QLinearArgs a) {
   return check_launch();
 }
 
-static bool four_wave(int K) { return K % 256 == 0 && K < 8192; }
+// Which kernel serves a projection: the 4-wave kernel needs K % 256 == 0; deep projections
+// (K >= 8192) and mid-width ones (40 to 191 column blocks: enough workgroups of 8 waves to fill
+// the CUs in one round; measured on the q|k|v shape) go to the k-way kernel.
+static bool four_wave_shape(int K) { return K % 256 == 0 && K < 8192; }
+static bool four_wave(int K, int N) {
+  const int nblocks = (N + 127) / 128;
+  return four_wave_shape(K) && !(nblocks >= 40 && nblocks < 192);
+}
 
 static int slice_len(int KT, int s) { return ((KT + s - 1) / s + 3) / 4 * 4; }
 static bool slices_ok(int KT, int s) { return (KT + slice_len(KT, s) - 1) / slice_len(KT, s) == s; }
@@ -696,7 +703,7 @@ static int num_splits4(int K, int N) {
 }
 
 int qlinear_num_splits(int K, int N, int M) {
-  if (four_wave(K)) return num_splits4(K, N);
+  if (four_wave(K, N)) return num_splits4(K, N);
   const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
   const int ks = M > 64 ? 4 : 8;
@@ -715,17 +722,17 @@ int qlinear_num_splits(int K, int N, int M) {
 // Number of K-slices of the LoRA projection t = x . A: as fine as whole steps (4 or 8 k-tiles,
 // by kernel) allow, at most TMX_MAX_LORA_SPLITS planes, so that no LoRA block outlasts the
 // main blocks.
-static int lora_step(int K) { return four_wave(K) ? 4 : 8; }
-int qlinear_num_lora_splits(int K) {
-  const int KT = K / 64, g = lora_step(K);
+static int lora_step(int K, int N) { return four_wave(K, N) ? 4 : 8; }
+int qlinear_num_lora_splits(int K, int N) {
+  const int KT = K / 64, g = lora_step(K, N);
   for (int per = g;; per += g) {
     const int n = (KT + per - 1) / per;
     if (n <= TMX_MAX_LORA_SPLITS) return n;
   }
 }
 
-static int lora_slice_len(int K) {
-  const int KT = K / 64, n = qlinear_num_lora_splits(K), g = lora_step(K);
+static int lora_slice_len(int K, int N) {
+  const int KT = K / 64, n = qlinear_num_lora_splits(K, N), g = lora_step(K, N);
   return ((KT + n - 1) / n + g - 1) / g * g;
 }
 
@@ -736,7 +743,7 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
                            int F, int G) {
   if (!x || !qw || !scales || !act) return TMX_ERR_ARG;
-  if (M <= 0 || M > 128 || !four_wave(K) || F % 64 || G % 64 || (G & (G - 1)) || K % G || ldx % 8)
+  if (M <= 0 || M > 128 || !four_wave_shape(K) || F % 64 || G % 64 || (G & (G - 1)) || K % G || ldx % 8)
     return TMX_ERR_SHAPE;
   if (a_t && (!lora_b || r <= 0 || 2 * r > 32)) return TMX_ERR_SHAPE;
   QLinearArgs a = {};
@@ -773,7 +780,7 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
 
 // Host-side dispatch shared by the C entry point and the decode-step launcher.
 // Output: y_bf16 [M, N] when nsplit == 1 and y_bf16 != null, else y_part
-// [nsplit][M][N] f32 planes.  t_part: [qlinear_num_lora_splits()][M][ldt] f32.
+// [nsplit][M][N] f32 planes.  t_part: [qlinear_num_lora_splits(K, N)][M][ldt] f32.
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
                  int N, int G, int Rpad, int nsplit) {
@@ -799,10 +806,10 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   a.M = M; a.K = K; a.N = N; a.G = G; a.Rpad = Rpad;
   a.nsplit = nsplit;
   a.kt_per_split = slice_len(KT, nsplit);
-  const int nls = qlinear_num_lora_splits(K);
+  const int nls = qlinear_num_lora_splits(K, N);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
-  a.kt_per_lora_split = lora_slice_len(K);
-  if (four_wave(K)) {
+  a.kt_per_lora_split = lora_slice_len(K, N);
+  if (four_wave(K, N)) {
     if (M <= 32) return launch_qlinear4<1>(st, a);
     if (M <= 64) return launch_qlinear4<2>(st, a);
     return launch_qlinear4<4>(st, a);
@@ -886,7 +893,7 @@ extern "C" size_t tmx_qlora_linear_workspace_bytes(int M, int K, int N) {
 }
 
 extern "C" int tmx_qlora_linear_num_splits(int M, int K, int N) { return qlinear_num_splits(K, N, M); }
-extern "C" int tmx_qlora_linear_num_lora_splits(int K) { return qlinear_num_lora_splits(K); }
+extern "C" int tmx_qlora_linear_num_lora_splits(int K, int N) { return qlinear_num_lora_splits(K, N); }
 
 extern "C" int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight,
                                        const void* scales, const void* lora_a_t, float* y_part,
@@ -911,7 +918,7 @@ extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight
                         TMX_MAX_RPAD, M, K, N, G, r_pad, ns);
   if (rc != TMX_OK) return rc;
   hipLaunchKernelGGL(lora_apply_kernel, dim3((N + 255) / 256, M), dim3(256), 0, st, (uint16_t*)y, y_part,
-                     ns, lora ? t_part : nullptr, qlinear_num_lora_splits(K), TMX_MAX_RPAD,
+                     ns, lora ? t_part : nullptr, qlinear_num_lora_splits(K, N), TMX_MAX_RPAD,
                      (const uint16_t*)lora_b, r, lora_scale,
                      (const uint16_t*)residual, M, N);
   return check_launch();

@@ -184,7 +184,7 @@ int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void
 size_t nucleus_bytes(int M, int V);
 size_t head_partial_bytes(int M, int V);
 int qlinear_num_splits(int K, int N, int M);
-int qlinear_num_lora_splits(int K);
+int qlinear_num_lora_splits(int K, int N);
 int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
                            int F, int G);
