@@ -247,6 +247,11 @@ typedef struct {
   size_t workspace_bytes;
   void* nucleus_workspace; /* tmx_nucleus_workspace_bytes(B, V); needed when top_p < 1 or top_k > 0 */
   size_t nucleus_workspace_bytes;
+  int tokens_per_pass;     /* 0 or 1: one token per sequence and step.  T > 1 (cache fill with
+                              sample == 0, or TMX_SAMPLE_SCORE): every pass consumes the T tokens at
+                              columns *step .. *step + T - 1 of each sequence as batch * T rows (<= 128),
+                              each attending to the slots up to its own column; *step advances by T.
+                              The workspace must be sized for batch * T rows. */
 } tmx_decode_state;
 
 size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int cache_size);

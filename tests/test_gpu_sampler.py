@@ -354,3 +354,52 @@ def test_per_token_logps_match_oracle_and_the_rollout_logprobs():
   np.testing.assert_allclose(scored, np.stack(ro.logprobs), atol=2e-5)
   with pytest.raises(ValueError):
     s.per_token_logps(np.zeros((2, 0), np.int32), comp[:2])
+
+
+@pytest.mark.parametrize('family', ['llama3', 'qwen3', 'moe'])
+def test_multi_token_passes_equal_one_token_passes(family):
+  """Cache fill and scoring in passes of several tokens per sequence (rows = sequences x tokens)
+  against the one-token walk: same KV cache, same next-step logits, same per-token log-probs up
+  to the f32 summation order of differently split projections."""
+  if family == 'moe':
+    cfg = OM.Config('qwen3', 2, 1024, 256, 256, 4, 64, 2, rope_theta=1_000_000, norm_eps=1e-6, tied=False,
+                    num_experts=8, experts_per_tok=2)
+  elif family == 'qwen3':
+    cfg = OM.Config('qwen3', 2, 1024, 256, 1024, 4, 64, 2, rope_theta=1_000_000, norm_eps=1e-6, tied=False)
+  else:
+    cfg = C.TOY
+  st0 = C.make_state(cfg, 41, 8, norm_jitter=0.05)
+  model = C.product_model(cfg, st0, 64, 16.0)
+  s = _sampler(model, cfg, 64)
+  s.eos_ids = np.array([-1])
+  rng = np.random.default_rng(3)
+  ids = rng.integers(3, cfg.vocab_size, (3, 41)).astype(np.int32)
+  ids[1, :7] = 0   # left padding
+  ids[2, :1] = 0
+  def fill(tokens_per_pass):
+    st = s.init_sample_state(ids, 48, True, None, 0.0, None, None, 0, include_logprobs=True)
+    n = 40
+    while n > 0:
+      t = min(tokens_per_pass, n)
+      s.run_steps(st, 1, sample=False, tokens_per_pass=t)
+      n -= t
+    assert int(st['step'].item()) == 40
+    cache = st['cache'].float().cpu().numpy().copy()
+    s.run_steps(st, 1, sample=True)
+    return cache, st['logits'].cpu().numpy().copy(), st['token_buffer'][:, 41].cpu().numpy().copy()
+  c1, l1, t1 = fill(1)
+  for tpp in (2, 7, 40):
+    c, l, t = fill(tpp)
+    assert np.abs(c - c1).max() <= 2.0 ** -6 * max(1.0, np.abs(c1).max()), tpp
+    assert np.abs(l - l1).max() <= LOGIT_TOL, (tpp, np.abs(l - l1).max())
+  # scoring: Sampler.per_token_logps walks in multi-token passes; compare with one token per pass
+  prompt, comp = ids[:, :20], ids[:, 20:]
+  got = s.per_token_logps(prompt, comp, pad_id=0)
+  s.MAX_ROWS = 3  # one token per sequence and pass
+  try:
+    one = s.per_token_logps(prompt, comp, pad_id=0)
+  finally:
+    s.MAX_ROWS = Sampler.MAX_ROWS
+  assert np.abs(got - one).max() <= LOGPROB_TOL, np.abs(got - one).max()
+  with pytest.raises(Exception):
+    s.run_steps(s.init_sample_state(ids, 48, False, None, 0.0, None, None, 0), 1, sample=True, tokens_per_pass=2)

@@ -51,7 +51,9 @@ __global__ __launch_bounds__(AttnWaves<G>::value * 64) void gqa_decode_kernel(At
   const int kvh = blockIdx.x, b = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int pg = lane / LPP, dl = lane % LPP;  // lane group, 8-element slice index
-  const int step = *a.step;
+  const int tpp = a.tpp > 0 ? a.tpp : 1;
+  const int seq = b / tpp;                    // b: query row of this pass
+  const int step = *a.step + b % tpp;
   // the splits share the VALID positions 0 .. step (not the cache size) in chunks of whole
   // 32 positions, so that every split has work at any context length
   const int chunk = (((step + a.nsplit) / a.nsplit) + 31) & ~31;
@@ -75,9 +77,9 @@ __global__ __launch_bounds__(AttnWaves<G>::value * 64) void gqa_decode_kernel(At
     for (int d = 0; d < 8; ++d) acc[g][d] = 0.f;
   }
   const size_t row_stride = (size_t)a.Kh * H;  // elements between consecutive positions
-  const uint16_t* kbase = a.kcache + ((size_t)b * a.C * a.Kh + kvh) * H + dl * 8;
-  const uint16_t* vbase = a.vcache + ((size_t)b * a.C * a.Kh + kvh) * H + dl * 8;
-  const uint8_t* mrow = a.input_mask + (size_t)b * a.buf_len;
+  const uint16_t* kbase = a.kcache + ((size_t)seq * a.C * a.Kh + kvh) * H + dl * 8;
+  const uint16_t* vbase = a.vcache + ((size_t)seq * a.C * a.Kh + kvh) * H + dl * 8;
+  const uint8_t* mrow = a.input_mask + (size_t)seq * a.buf_len;
 
   // lane group (wave, pg) takes positions s_begin + (it * NG + wave * PPW + pg) * U + u
   for (int p0 = s_begin + (wave * PPW + pg) * U; p0 < s_end; p0 += NG * U) {

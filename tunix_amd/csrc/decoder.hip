@@ -108,11 +108,16 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       !s->workspace)
     return TMX_ERR_ARG;
   const bool moe = m->num_experts > 0;
+  // rows of a pass: one per sequence, or tokens_per_pass consecutive tokens of every sequence
+  // (cache fill and scoring only: sampling needs the previous token)
+  const int NSEQ = s->batch, T = s->tokens_per_pass > 1 ? s->tokens_per_pass : 1;
+  if (NSEQ <= 0 || NSEQ > 128 || T > 128) return TMX_ERR_SHAPE;
+  if (T > 1 && sample && s->sampling_mode != TMX_SAMPLE_SCORE) return TMX_ERR_ARG;
+  const int B = NSEQ * T, C = s->cache_size, L = s->buf_len;
+  if (B > 128 || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
   if (moe && (m->experts_per_tok <= 0 || m->experts_per_tok > m->num_experts ||
-              (size_t)s->batch * m->experts_per_tok > 1024))
+              (size_t)B * m->experts_per_tok > 1024))
     return TMX_ERR_SHAPE;
-  const int B = s->batch, C = s->cache_size, L = s->buf_len;
-  if (B <= 0 || B > 128 || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
   const bool nucleus = sample && s->sampling_mode == TMX_SAMPLE_TOP_P && (s->top_p < 1.0f || s->top_k > 0);
   if (nucleus && !s->nucleus_workspace) return TMX_ERR_ARG;
   const int D = m->embed_dim, N = m->num_heads, Kh = m->num_kv_heads, H = m->head_dim;
@@ -131,7 +136,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   }
   hipStream_t st = (hipStream_t)stream;
   const Workspace w = carve(m, B, C, (char*)s->workspace);
-  const size_t kv_elems = (size_t)B * C * Kh * H;
+  const size_t kv_elems = (size_t)NSEQ * C * Kh * H;
   const float theta = m->family == TMX_FAMILY_LLAMA3 ? 1000000.0f : m->rope_theta;
   int rc;
 #define TMX_TRY(kind, expr)            \
@@ -162,6 +167,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       a.token_buffer = s->token_buffer;
       a.step = s->step;
       a.buf_len = L;
+      a.tpp = T;
       a.positions = s->positions;
       a.rope_tab = w.rope_tab;
       a.half = H / 2;
@@ -189,7 +195,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         a.lora = lora_of(l.qkv, sp.qkv);
         a.q_norm_w = (const uint16_t*)l.q_norm_w;
         a.k_norm_w = (const uint16_t*)l.k_norm_w;
-        a.positions = s->positions; a.step = s->step; a.buf_len = L;
+        a.positions = s->positions; a.step = s->step; a.buf_len = L; a.tpp = T;
         a.rope_tab = w.rope_tab;
         a.q_out = w.q; a.kcache = kc; a.vcache = vc;
         a.N = N; a.Kh = Kh; a.H = H; a.C = C;
@@ -199,7 +205,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       {
         AttnArgs a = {};
         a.q = w.q; a.kcache = kc; a.vcache = vc;
-        a.input_mask = s->input_mask; a.step = s->step; a.buf_len = L;
+        a.input_mask = s->input_mask; a.step = s->step; a.buf_len = L; a.tpp = T;
         a.out = w.attn; a.partial = w.attn_partial;
         a.B = B; a.N = N; a.Kh = Kh; a.C = C;
         a.scale = 1.0f / sqrtf((float)H);
@@ -305,6 +311,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       a.done = s->done;
       a.eos = s->eos_ids; a.n_eos = s->n_eos;
       a.buf_len = L;
+      a.tpp = T;
       if (nucleus) {
         TMX_TRY(TMX_K_HEAD, head_sample_nucleus(st, a, s->top_p, s->top_k, s->nucleus_workspace,
                                                 s->nucleus_workspace_bytes));
@@ -312,7 +319,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         TMX_TRY(TMX_K_HEAD, head_sample(st, a));
       }
     }
-    TMX_TRY(TMX_K_ADVANCE, advance_step(st, s->step));
+    TMX_TRY(TMX_K_ADVANCE, advance_step(st, s->step, T));
   }
 #undef TMX_TRY
   return TMX_OK;

@@ -145,11 +145,12 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
   float ss = 0.f;
   const uint16_t* src = nullptr;
   if (a.embed) {
-    const int step = *a.step;
-    const int tok = a.token_buffer[(size_t)m * a.buf_len + step];
+    const int tpp = a.tpp > 0 ? a.tpp : 1;
+    const int seq = m / tpp, step = *a.step + m % tpp;
+    const int tok = a.token_buffer[(size_t)seq * a.buf_len + step];
     src = a.embed + (size_t)tok * a.D;
     if (a.rope_tab && (int)threadIdx.x < a.half) {
-      const float pos = (float)a.positions[(size_t)m * a.buf_len + step];
+      const float pos = (float)a.positions[(size_t)seq * a.buf_len + step];
       const float frac = 2.f * (float)threadIdx.x / (float)(2 * a.half);
       const float ang = pos / powf(a.theta, frac);
       a.rope_tab[((size_t)m * a.half + threadIdx.x) * 2] = sinf(ang);
@@ -245,7 +246,8 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
   __shared__ float t_s[64];
   const int head = blockIdx.x, b = blockIdx.y, B = gridDim.y, lane = threadIdx.x;
   const int half = a.H >> 1;
-  const int step = *a.step;
+  const int tpp = a.tpp > 0 ? a.tpp : 1;
+  const int seq = b / tpp, step = *a.step + b % tpp;  // b: row of this pass
   const bool active = lane < half;
   const int ntot = (a.N + 2 * a.Kh) * a.H;
   const int kind = head < a.N ? 0 : (head < a.N + a.Kh ? 1 : 2);  // q, k, v
@@ -278,7 +280,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
   const int slot = step % a.C;
   if (kind == 2) {
     if (active) {
-      uint16_t* dst = a.vcache + (((size_t)b * a.C + slot) * a.Kh + (head - a.N - a.Kh)) * a.H;
+      uint16_t* dst = a.vcache + (((size_t)seq * a.C + slot) * a.Kh + (head - a.N - a.Kh)) * a.H;
       dst[lane] = f2bf(x1);
       dst[lane + half] = f2bf(x2);
     }
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
       sn = a.rope_tab[((size_t)b * half + lane) * 2];
       cs = a.rope_tab[((size_t)b * half + lane) * 2 + 1];
     } else {
-      const float pos = (float)a.positions[(size_t)b * a.buf_len + step];
+      const float pos = (float)a.positions[(size_t)seq * a.buf_len + step];
       const float ang = pos / powf(a.theta, 2.f * (float)lane / (float)a.H);
       sn = sinf(ang);
       cs = cosf(ang);
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
     }
     uint16_t* dst;
     if (kind == 0) dst = a.q_out + (size_t)b * a.N * a.H + head * a.H;
-    else dst = a.kcache + (((size_t)b * a.C + slot) * a.Kh + (head - a.N)) * a.H;
+    else dst = a.kcache + (((size_t)seq * a.C + slot) * a.Kh + (head - a.N)) * a.H;
     dst[lane] = f2bf(o1);
     dst[lane + half] = f2bf(o2);
   }
@@ -364,12 +366,12 @@ int swiglu(hipStream_t st, const SwigluArgs& a, int M) {
   return check_launch();
 }
 
-// step += 1 (one thread); keeps the step counter on the device so that a captured
+// step += tokens per pass (one thread); keeps the step counter on the device so that a captured
 // graph of one decode step can be replayed without host-side parameters.
-__global__ void advance_step_kernel(int32_t* step) { *step += 1; }
+__global__ void advance_step_kernel(int32_t* step, int by) { *step += by; }
 
-int advance_step(hipStream_t st, int32_t* step) {
-  hipLaunchKernelGGL(advance_step_kernel, dim3(1), dim3(1), 0, st, step);
+int advance_step(hipStream_t st, int32_t* step, int by) {
+  hipLaunchKernelGGL(advance_step_kernel, dim3(1), dim3(1), 0, st, step, by);
   return check_launch();
 }
 

@@ -134,7 +134,9 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     const int row = m * 32 + nl;
-    target[m] = (score && row < a.M) ? a.token_buffer[(size_t)row * a.buf_len + *a.step + 1] : -1;
+    const int tpp = a.tpp > 0 ? a.tpp : 1;
+    target[m] = (score && row < a.M)
+                    ? a.token_buffer[(size_t)(row / tpp) * a.buf_len + *a.step + row % tpp + 1] : -1;
   }
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
@@ -245,11 +247,13 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
       Best o = {s_f[w][2], s_f[w][3], s_i[w]};
       best_merge(best, o);
     }
-    const int col = *a.step + 1;
     if (a.mode == TMX_SAMPLE_SCORE) {  // teacher forcing: the token stays, only its log-prob is written
-      if (a.logprobs) a.logprobs[(size_t)row * a.buf_len + col] = (best.z - mx) - logf(se);
+      const int tpp = a.tpp > 0 ? a.tpp : 1;
+      if (a.logprobs)
+        a.logprobs[(size_t)(row / tpp) * a.buf_len + *a.step + row % tpp + 1] = (best.z - mx) - logf(se);
       return;
     }
+    const int col = *a.step + 1;
     const int tok = best.idx;
     a.token_buffer[(size_t)row * a.buf_len + col] = tok;
     if (a.logprobs) a.logprobs[(size_t)row * a.buf_len + col] = (best.z - mx) - logf(se);

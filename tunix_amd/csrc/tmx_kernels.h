@@ -66,6 +66,7 @@ struct RowNormArgs {
   const int32_t* token_buffer;  // [B, L]
   const int32_t* step;          // device scalar: column of token_buffer to read
   int buf_len;
+  int tpp;                      // tokens per pass: row m is sequence m / tpp at column *step + m % tpp (0: 1)
   const int32_t* positions;     // [B, L] (embedding mode: fills rope_tab)
   float* rope_tab;              // [B][half][2] sin, cos of this step (may be null)
   int half;
@@ -96,6 +97,7 @@ struct RopeArgs {
   const int32_t* positions;  // [B, L]
   const int32_t* step;
   int buf_len;
+  int tpp;                   // tokens per pass (0: 1): row m is sequence m / tpp at slot *step + m % tpp
   const float* rope_tab;     // [B][H/2][2] or null (then sin/cos are computed here)
   uint16_t* q_out;           // [B, N * H]
   uint16_t* kcache;          // [B, C, Kh, H]
@@ -125,6 +127,7 @@ struct AttnArgs {
   float* partial;    // [B, Kh, nsplit, G, H + 2] (nsplit > 1)
   int B, N, Kh, C, nsplit, chunk;
   float scale;
+  int tpp;  // tokens per pass (0: 1): query row m belongs to sequence m / tpp and sees slots <= *step + m % tpp
 };
 
 struct HeadArgs {
@@ -149,6 +152,7 @@ struct HeadArgs {
   const int32_t* eos;
   int n_eos;
   int buf_len;
+  int tpp;  // tokens per pass (0: 1), score mode only: row m is sequence m / tpp at column *step + m % tpp
 };
 
 
@@ -172,7 +176,7 @@ struct NucleusArgs {
 int row_norm(hipStream_t st, const RowNormArgs& a, int M);
 int rope_kvwrite(hipStream_t st, const RopeArgs& a, int B);
 int swiglu(hipStream_t st, const SwigluArgs& a, int M);
-int advance_step(hipStream_t st, int32_t* step);
+int advance_step(hipStream_t st, int32_t* step, int by);
 int empty_launch(hipStream_t st);  // measurement aid: a kernel that does nothing
 int gqa_decode(hipStream_t st, AttnArgs a, int H);
 size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);

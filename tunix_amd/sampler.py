@@ -188,13 +188,14 @@ class Sampler:
     }
     return st
 
-  def _c_state(self, st):
+  def _c_state(self, st, tokens_per_pass=1):
     b, total = st['token_buffer'].shape
     ws_bytes = self._lib.tmx_decode_workspace_bytes(
-        ctypes.byref(self._transformer.desc()), b, self.cache_config.cache_size)
+        ctypes.byref(self._transformer.desc()), b * tokens_per_pass, self.cache_config.cache_size)
     if self._workspace is None or self._workspace.numel() < ws_bytes:
       self._workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=self._transformer.device)
     s = DecodeState()
+    s.tokens_per_pass = tokens_per_pass
     s.batch, s.buf_len, s.cache_size = b, total, self.cache_config.cache_size
     s.token_buffer, s.positions = st['token_buffer'].data_ptr(), st['positions'].data_ptr()
     s.input_mask, s.done, s.step = st['input_mask'].data_ptr(), st['done'].data_ptr(), st['step'].data_ptr()
@@ -220,12 +221,27 @@ class Sampler:
       s.nucleus_workspace, s.nucleus_workspace_bytes = self._nucleus_ws.data_ptr(), self._nucleus_ws.numel()
     return s
 
-  def run_steps(self, st, n_steps, sample=True, graph=False):
+  MAX_ROWS = 128  # rows of one pass the kernels take (sequences x tokens per pass)
+
+  def walk(self, st, n_tokens, sample=False):
+    """Advances every sequence by n_tokens known tokens (cache fill over a prompt, or scoring
+    when st['sampling_mode'] == 'score') in passes of as many tokens per sequence as fit
+    MAX_ROWS rows, instead of one token per launch sequence."""
+    b = st['token_buffer'].shape[0]
+    per = max(1, self.MAX_ROWS // b)
+    while n_tokens > 0:
+      t = min(per, n_tokens)
+      self.run_steps(st, 1, sample=sample, tokens_per_pass=t)
+      n_tokens -= t
+
+  def run_steps(self, st, n_steps, sample=True, graph=False, tokens_per_pass=1):
     """Runs n decode-loop iterations on the current stream.  graph=False only enqueues (no host
-    sync); graph=True replays one recorded step and returns when the steps have run."""
+    sync); graph=True replays one recorded step and returns when the steps have run.
+    tokens_per_pass > 1: every iteration consumes that many known tokens of each sequence
+    (cache fill or scoring only)."""
     if n_steps <= 0:
       return
-    cs = self._c_state(st)
+    cs = self._c_state(st, tokens_per_pass)
     fn = self._lib.tmx_decode_steps_graph if graph else self._lib.tmx_decode_steps
     rc = fn(ctypes.byref(self._transformer.desc()), ctypes.byref(cs), _lib.stream(), int(n_steps),
             1 if sample else 0)
@@ -264,8 +280,8 @@ class Sampler:
     st['input_mask'] = torch.from_numpy(valid.astype(np.uint8)).to(dev)
     st['positions'] = torch.from_numpy(utils.build_positions_from_mask(valid).astype(np.int32)).to(dev)
     st['sampling_mode'] = 'score'
-    self.run_steps(st, p - 1, sample=False)
-    self.run_steps(st, t, sample=True)
+    self.walk(st, p - 1)
+    self.walk(st, t, sample=True)
     return st['logprobs'][:, p:p + t].cpu().numpy()
 
   # -- the call ---------------------------------------------------------------
@@ -301,7 +317,7 @@ class Sampler:
     logits_steps = []
     if max_generation_steps > 0:
       # cache fill over prompt columns 0 .. P-2, then P-1 produces generated token #1
-      self.run_steps(st, p - 1, sample=False, graph=self.use_graph)
+      self.walk(st, p - 1)
       remaining = max_generation_steps
       while remaining > 0:
         n = 1 if return_logits else min(self.CHECK_EVERY, remaining)
