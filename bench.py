@@ -282,7 +282,11 @@ def main():
       gu = layer0['gate_up']
       fused = (tot_cnt[CLASS_NAMES.index('swiglu')] == 0 and gu.k % 256 == 0 and gu.k < 8192)
       if fused:
-        sym = f'tmx::qlinear_gate_up_kernel<{mt}>' if gu.lora_a_t is not None else f'tmx::qlinear_mfma4_kernel<{mt}>'
+        lora = gu.lora_a_t is not None
+        if batch <= 64 and gu.k % 512 == 0:   # 8 waves per workgroup, activation slab by direct-to-LDS loads
+          sym = f"tmx::qlinear_gate_up8_kernel<{mt}, {'true' if lora else 'false'}>"
+        else:
+          sym = f'tmx::qlinear_gate_up_kernel<{mt}>' if lora else f'tmx::qlinear_mfma4_kernel<{mt}>'
         symbols.setdefault(sym, []).append('gate_up_linear')
       else:
         dense.append(('gate_up_linear', 'gate_up'))

@@ -125,6 +125,15 @@ int tmx_swiglu(void* stream, const void* gate_up_bf16, const float* gate_up_part
                const float* t_part, int t_nsplit, int ldt, const void* lora_b, int r, float lora_scale,
                void* act, int M, int F);
 
+/* act[M, F] = bf16(silu(g) * u) with g | u = x . dequant(Wq, s) (+ LoRA deltas) for the stacked
+ * gate | up matrix [K, 2F], in one launch: projection, LoRA and SwiGLU fused.  Needs
+ * K % 256 == 0, K < 8192, F % 64 == 0; with LoRA lora_a_t = [A_gate | A_up] in fragment order
+ * with r_pad == 32 (2 r <= 32) and lora_b [r][2F].  tunix/models/llama3/model.py:489-496 with
+ * the qwix-wrapped projections of :461-487. */
+int tmx_qlora_gate_up_swiglu(void* stream, const void* x, const void* qweight, const void* scales,
+                             const void* lora_a_t, const void* lora_b, void* act, int M, int K, int F,
+                             int G, int r, float lora_scale);
+
 /* ---- GQA decode attention -------------------------------------------------- */
 
 /* out[B, N H] = softmax(q . K^T / sqrt(H) over positions j <= *step with

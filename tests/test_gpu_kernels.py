@@ -212,6 +212,43 @@ def test_swiglu(M, F, ns):
   G.assert_bf16_close(G.host(act), ref, ulps=1.0, min_exact=0.98, what='swiglu')
 
 
+@pytest.mark.parametrize('M,K,F,group,r', [
+    (4, 256, 128, 64, 8), (33, 768, 192, 64, 0), (64, 512, 256, 64, 16), (17, 1024, 320, 128, 16),
+    (64, 2048, 1024, 64, 0), (40, 4096, 512, 64, 16), (100, 1024, 256, 64, 8), (128, 512, 128, 128, 0),
+])
+def test_fused_gate_up_swiglu_matches_oracle(M, K, F, group, r):
+  """One launch for gate | up + LoRA + SwiGLU against the oracle's separate projections (K in
+  multiples of 512 up to 64 rows runs the 8-wave kernel, the rest the 4-wave one)."""
+  rng = np.random.default_rng(M + K + F)
+  x = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+  ws = [bf16_round(rng.standard_normal((K, F)).astype(np.float32) * 0.03) for _ in range(2)]
+  loras = None
+  if r:
+    loras = [(bf16_round(rng.standard_normal((K, r)).astype(np.float32) * 0.03),
+              bf16_round(rng.standard_normal((r, F)).astype(np.float32) * 0.03)) for _ in range(2)]
+  pl = quant.PackedLinear.from_dense([torch.from_numpy(w) for w in ws], group, G.DEV,
+                                     None if loras is None else [tuple(torch.from_numpy(m) for m in l) for l in loras],
+                                     2.0)
+  ys = []
+  for i, w in enumerate(ws):
+    qo, so = int4.quantize(w, group)
+    lin = L.Linear(q=qo, scale=so, group=group, a=loras[i][0] if r else None, b=loras[i][1] if r else None,
+                   lora_scale=2.0)
+    ys.append(lin(x, BF16))
+  ref = bf16_round(L.silu(ys[0], BF16) * ys[1])
+  xt = G.bf(x)
+  act = torch.empty(M, F, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_qlora_gate_up_swiglu', S(), G.p(xt), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t),
+         G.p(pl.lora_b), G.p(act), M, K, F, group, r, 2.0)
+  G.sync()
+  # a one-ulp flip of g or u (f32 summation order) moves the product by about one ulp of it,
+  # silu' <= 1.1 adds a little, and both can flip; rare
+  extra = 2.5 * np.maximum(G.ulp_bf16(ref), G.ulp_bf16(ys[0]) * np.abs(ys[1]))
+  G.assert_bf16_close(G.host(act), ref, ulps=1.0, extra=extra, min_exact=0.97, what=f'gate_up {M}x{K}x{F}')
+  assert _lib.lib().tmx_qlora_gate_up_swiglu(S(), G.p(xt), G.p(pl.qweight), G.p(pl.scales), None, None, G.p(act),
+              M, K, F + 32, group, 0, 0.0) != 0
+
+
 @pytest.mark.parametrize('B,N,Kh,H,C,step', [
     (2, 4, 4, 64, 64, 40), (3, 8, 2, 64, 96, 95), (2, 8, 4, 64, 33, 0), (4, 32, 8, 128, 300, 257),
     (2, 8, 1, 128, 128, 100), (1, 32, 8, 64, 768, 700), (2, 16, 8, 128, 520, 519), (1, 4, 4, 128, 16, 7),

@@ -38,7 +38,7 @@ def build(verbose=False, jobs=6):
   with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
     outs = list(ex.map(lambda so: _run([hipcc] + HIPCC_FLAGS + inc + ['-c', so[0], '-o', so[1]]),
                        zip(srcs, objs)))
-  outs.append(_run([hipcc, '--offload-arch=gfx950', '-shared', '-fPIC', '-o', LIB_PATH] + objs))
+  outs.append(_run([hipcc, '--offload-arch=gfx950', '-shared', '-fPIC', '-Wl,--no-undefined', '-o', LIB_PATH] + objs))
   if verbose:
     print('\n'.join(o for o in outs if o.strip()))
   return LIB_PATH

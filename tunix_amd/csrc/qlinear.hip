@@ -16,43 +16,6 @@
 
 namespace tmx {
 
-// Expand one 32-bit word (8 nibbles, element j = 2 (i % 4) + i / 4 for nibble i)
-// into the 8 bf16 B-operand values of one MFMA step: bf16((u - 8) * s).
-__device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s) {
-  uint32_t lo = d & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
-  uint32_t hi = (d >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7 in bytes 0..3
-  // keep the two masked words opaque so that each byte is widened by one
-  // v_cvt_f32_ubyteN instead of a bit-field extract plus a conversion
-  asm volatile("" : "+v"(lo), "+v"(hi));
-  // nibble i: byte i/2 of (i even ? lo : hi)
-  const float n0 = (float)(lo & 0xFF), n1 = (float)(hi & 0xFF);
-  const float n2 = (float)((lo >> 8) & 0xFF), n3 = (float)((hi >> 8) & 0xFF);
-  const float n4 = (float)((lo >> 16) & 0xFF), n5 = (float)((hi >> 16) & 0xFF);
-  const float n6 = (float)(lo >> 24), n7 = (float)(hi >> 24);
-  // register p holds elements j = 2p, 2p + 1  <->  nibbles p, p + 4
-  uint32_t p[4];
-  p[0] = pack_bf2(fmaf(n0, s, m8s), fmaf(n4, s, m8s));
-  p[1] = pack_bf2(fmaf(n1, s, m8s), fmaf(n5, s, m8s));
-  p[2] = pack_bf2(fmaf(n2, s, m8s), fmaf(n6, s, m8s));
-  p[3] = pack_bf2(fmaf(n3, s, m8s), fmaf(n7, s, m8s));
-  bf16x8_t b;
-  __builtin_memcpy(&b, p, 16);
-  return b;
-}
-
-
-template <int V>
-struct IC { static constexpr int value = V; };
-
-// f(IC<0>{}), ..., f(IC<N - 1>{}): a loop whose index is a compile-time constant
-template <int N, int I = 0, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (I < N) {
-    f(IC<I>{});
-    static_for<N, I + 1>(f);
-  }
-}
-
 // Two kernels share the tile math.  The 4-wave kernel (one wave per column tile, steps of 4
 // k-tiles) serves K % 256 == 0 below 8192; the k-way kernel further down runs two waves per
 // column tile over steps of 8 k-tiles, takes any K % 64 == 0 and serves the deep projections.
@@ -671,6 +634,277 @@ static int launch_qlinear(hipStream_t st, QLinearArgs a) {
   return check_launch();
 }
 
+// ---------------------------------------------------------------------------
+// gate | up with SwiGLU (and LoRA) in the epilogue, 8 waves per workgroup.  The workgroup owns
+// 2 gate tiles and the 2 matching up tiles like the 4-wave pair block, but two waves share each
+// column tile: wave (cw, kh) multiplies tile cw by k-tiles kh * TPW .. kh * TPW + TPW - 1 of
+// every step (starting at k-tile kh * TPW + cw, the one whose LoRA product x . A it also owns), so each SIMD holds two waves whose dequantisation, MFMA and load waits overlap.
+// All global reads are buffer loads: a per-lane byte offset that never changes plus a scalar
+// offset that advances per step, so the loop carries no per-lane address arithmetic.
+template <int MT>
+struct GU8 {
+  static constexpr int TS = 8;                 // k-tiles per step
+  static constexpr int TPW = TS / 2;           // k-tiles per wave and step
+  static constexpr int XS = TS * 64 + 8;       // bf16 elements per LDS row
+  static constexpr int ROWS = MT * 32;
+  static constexpr size_t SLAB = (size_t)2 * ROWS * XS * 2;
+  static constexpr size_t EPI = (size_t)8 * MT * 16 * 64 * 4 + (size_t)ROWS * 40 * 2;
+  static constexpr size_t LDS = SLAB > EPI ? SLAB : EPI;
+};
+
+
+
+template <int MT, bool FUSE>
+__global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a) {
+  using S = GU8<MT>;
+  constexpr int TS = S::TS, TPW = S::TPW, XS = S::XS, ROWS = S::ROWS;
+  extern __shared__ __align__(16) uint16_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), cw = wave & 3, kh = wave >> 2;
+  const int h = lane >> 5, nl = lane & 31;
+  const int KT = a.K >> 6, nsteps = KT / TS, last_step = nsteps - 1;  // host: K % (64 TS) == 0
+  const int gs = __builtin_ctz(a.G >> 6), KG = a.K / a.G;
+  const int nb = (int)blockIdx.x * 2 + (cw & 1) + (cw >> 1) * a.pair_off;  // host: F % 64 == 0
+  TMX_STAMP(0);
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qw, (uint32_t)(a.N >> 5) * KT * 1024u);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scales, (uint32_t)(a.N >> 5) * KG * 64u);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, (uint32_t)a.M * a.ldx * 2u);
+  const __amdgpu_buffer_rsrc_t rl = make_rsrc(FUSE ? a.a_t : a.x, FUSE ? (uint32_t)KT * 4096u : 16u);
+  const int wv = (nb * KT * 64 + lane) * 16;  // per-lane byte offsets
+  const int sv = (nb * KG * 32 + nl) * 2;
+  const int lv = lane * 64;
+
+  f32x16_t acc[MT], tacc[FUSE ? MT : 1];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
+  if constexpr (FUSE) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tacc[m][r] = 0.f;
+  }
+
+  // activation slab of a step: one row (TS * 64 bf16 = 1 KiB) per direct-to-LDS load, rows
+  // wave, wave + 8, ... of the slab; the global address is wave-uniform apart from lane * 16
+  constexpr int XR = ROWS / 8;  // rows per wave and step
+  const int xv = lane * 16;
+  int xrow_off[XR];             // byte offset of each of this wave's rows (rows past M repeat the last)
+#pragma unroll
+  for (int i = 0; i < XR; ++i) {
+    const int row_l = wave + 8 * i;
+    xrow_off[i] = (row_l < a.M ? row_l : a.M - 1) * a.ldx * 2;
+  }
+  u32x4_t wring[2][TPW];
+  uint16_t sring[2][TPW];
+  u32x4_t lring[FUSE ? 2 : 1][4];
+
+  auto load_w_tile = [&](int step, auto dc, auto jc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+    step = step < last_step ? step : last_step;
+    const int kt = step * TS + kh * TPW + ((j + cw) & (TPW - 1));
+    wring[d][j] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv, kt * 1024, 0);
+    sring[d][j] = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
+  };
+  // global -> LDS without passing through registers (buffer_load ... lds: lane i lands at
+  // base + 16 i, so a row of the slab arrives contiguously and the 16-byte row pad is skipped)
+  auto dma_x = [&](int step, int buf) __attribute__((always_inline)) {
+    step = step < last_step ? step : last_step;
+    uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * XS;
+#pragma unroll
+    for (int i = 0; i < XR; ++i)
+      load_row_to_lds(rx, base + i * 8 * XS, xv, xrow_off[i] + step * (TS * 128));
+  };
+  auto load_l = [&](int step, auto dc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value;
+    step = step < last_step ? step : last_step;
+    const int so = (step * TS + kh * TPW + cw) * 4096;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) lring[d][t] = __builtin_amdgcn_raw_buffer_load_b128(rl, lv + t * 16, so, 0);
+  };
+  auto tile_math = [&](int step, int buf, auto dc, auto jc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kh * TPW + ((j + cw) & (TPW - 1))) * 64 + h * 8 + nl * XS;
+    bf16x8_t xa[MT][4];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + t * 16);
+    const u32x4_t wc = wring[d][j];
+    const float s_c = bf2f(sring[d][j]);
+    load_w_tile(step + 2, dc, jc);  // slot consumed: refill it two steps ahead
+    const float m8s = -8.f * s_c;
+    const uint32_t wd[4] = {wc.x, wc.y, wc.z, wc.w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const bf16x8_t b = dequant_word(wd[t], s_c, m8s);
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[m], 0, 0, 0);
+    }
+    if constexpr (FUSE && j == 0) {  // the wave's first k-tile of a step is kh * TPW + cw: its LoRA share
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const bf16x8_t b = __builtin_bit_cast(bf16x8_t, lring[d][t]);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+          tacc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, tacc[m], 0, 0, 0);
+      }
+      load_l(step + 2, dc);
+    }
+  };
+  // Loads of a step younger than its slab transfer: a weight tile and a scale per k-tile plus the
+  // four LoRA fragments of the duty tile.  s_waitcnt vmcnt(that count) therefore waits for the
+  // slab (in-order counter) while the weight prefetch stays in flight.
+  constexpr int kYounger = TPW * 2 + (FUSE ? 4 : 0);
+  static_assert(TPW == 4, "every wave has exactly one LoRA duty tile per step");
+  auto do_step = [&](int step, auto sc) __attribute__((always_inline)) {
+    constexpr int sp = decltype(sc)::value;
+    dma_x(step + 1, sp ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<TPW>([&](auto jc) __attribute__((always_inline)) { tile_math(step, sp, IC<sp>{}, jc); });
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
+    __syncthreads();
+  };
+
+  dma_x(0, 0);
+  static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(0, IC<0>{}, jc); });
+  static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(1, IC<1>{}, jc); });
+  if constexpr (FUSE) {
+    load_l(0, IC<0>{});
+    load_l(1, IC<1>{});
+  }
+  TMX_STAMP(1);
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | ((TPW * 4 + (FUSE ? 8 : 0)) & 15) | (((TPW * 4 + (FUSE ? 8 : 0)) >> 4) << 14));
+  __syncthreads();
+  TMX_STAMP(2);
+  const int npairs = nsteps / 2;
+  for (int g = 0; g < npairs; ++g) {
+    do_step(2 * g, IC<0>{});
+    TMX_STAMP(3 + 2 * g);
+    do_step(2 * g + 1, IC<1>{});
+    TMX_STAMP(4 + 2 * g);
+  }
+  if (nsteps & 1) do_step(nsteps - 1, IC<0>{});
+  TMX_STAMP(29);
+
+  // ---- epilogue (the slab is free: the last step ended with a barrier) ----
+  float* fl = reinterpret_cast<float*>(smem);
+  f32x16_t dl[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dl[m][r] = 0.f;
+  if constexpr (FUSE) {
+    // B fragment of this tile's columns (rows beyond the rank are zero, which also masks the t
+    // columns of the other projection inside the 16-wide k window); fetched before the barriers
+    // below so that the cold reads overlap them
+    bf16x8_t tb;
+    {
+      const int colw = nb * 32 + nl;
+      float bv[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = h * 8 + j;
+        bv[j] = k < a.lora_r ? bf2f(a.lora_b[(size_t)k * a.N + colw]) : 0.f;
+      }
+      uint32_t pb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pb[j] = pack_bf2(bv[2 * j], bv[2 * j + 1]);
+      __builtin_memcpy(&tb, pb, 16);
+    }
+    // 1. t = x . [A_gate | A_up]: the partial tiles of all waves meet in LDS, are summed in wave
+    // order, rounded to bf16 and laid out row-major for the MFMA A fragments of step 2
+    uint16_t* ts = reinterpret_cast<uint16_t*>(fl + 8 * MT * 16 * 64);  // [ROWS][40]
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) fl[(((wave * MT + m) * 16 + r) << 6) + lane] = tacc[m][r];
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr) {
+        const int r = wave * 2 + rr;
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) t += fl[(((w * MT + m) * 16 + r) << 6) + lane];
+        ts[(m * 32 + acc_row(r, lane)) * 40 + nl] = f2bf(t);
+      }
+    __syncthreads();
+    if (kh == 0) {
+      // 2. delta = t . B on the MFMA
+      const int toff = (cw >= 2) ? a.lora_r : 0;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        uint16_t tv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tv[j] = ts[(m * 32 + nl) * 40 + toff + h * 8 + j];
+        bf16x8_t ta;
+        __builtin_memcpy(&ta, tv, 16);
+        dl[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta, tb, dl[m], 0, 0, 0);
+      }
+    }
+    __syncthreads();  // ts / partial tiles are overwritten below
+  }
+  // the second k-half hands its accumulators to the first
+  if (kh == 1) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) fl[(((cw * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
+  }
+  __syncthreads();
+  if (kh == 0) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float y = rbf(acc[m][r] + fl[(((cw * MT + m) * 16 + r) << 6) + lane]);
+        if (FUSE) y = rbf(y + rbf(rbf(dl[m][r]) * a.lora_ls));
+        acc[m][r] = y;
+      }
+  }
+  __syncthreads();
+  // act = bf16(bf16(g * bf16(sigmoid(g))) * u): the up waves hand their tile to the gate waves
+  if (kh == 0 && cw >= 2) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) fl[((((cw - 2) * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
+  }
+  __syncthreads();
+  if (kh == 0 && cw < 2) {
+    const int col = ((int)blockIdx.x * 2 + cw) * 32 + nl;
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m * 32 + acc_row(r, lane);
+        if (row >= a.M) continue;
+        const float g = acc[m][r], u = fl[(((cw * MT + m) * 16 + r) << 6) + lane];
+        const float sg = rbf(1.f / (1.f + expf(-g)));
+        a.y_bf16[(size_t)row * a.ldy + col] = f2bf(rbf(g * sg) * u);
+      }
+  }
+  TMX_STAMP(30);
+}
+
+template <int MT, bool FUSE>
+static int launch_gate_up8(hipStream_t st, const QLinearArgs& a) {
+  using S = GU8<MT>;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&qlinear_gate_up8_kernel<MT, FUSE>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS);
+  if (attr != hipSuccess) return TMX_ERR_LAUNCH;
+  hipLaunchKernelGGL((qlinear_gate_up8_kernel<MT, FUSE>), dim3(a.n_main_blocks, 1), dim3(512), S::LDS, st, a);
+  return check_launch();
+}
+
 // Which kernel serves a projection: the 4-wave kernel needs K % 256 == 0; deep projections
 // (K >= 8192) and mid-width ones (40 to 191 column blocks: enough workgroups of 8 waves to fill
 // the CUs in one round; measured on the q|k|v shape) go to the k-way kernel.
@@ -768,6 +1002,12 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
     hipLaunchKernelGGL(kern, dim3(a.n_main_blocks, 1), dim3(256), 0, st, a);
     return check_launch();
   };
+  // up to 64 rows: 8 waves per workgroup, when steps of 8 k-tiles divide K and 32-bit byte
+  // offsets reach every operand (128 rows would not fit the register file at 2 waves per SIMD)
+  if (M <= 64 && K % 512 == 0 && (size_t)M * ldx * 2 < (1u << 31) && (size_t)K * F < (1u << 31)) {
+    if (a_t) return M <= 32 ? launch_gate_up8<1, true>(st, a) : launch_gate_up8<2, true>(st, a);
+    return M <= 32 ? launch_gate_up8<1, false>(st, a) : launch_gate_up8<2, false>(st, a);
+  }
   if (a_t) {
     if (M <= 32) return launch(qlinear_gate_up_kernel<1>);
     if (M <= 64) return launch(qlinear_gate_up_kernel<2>);
@@ -922,4 +1162,11 @@ extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight
                      (const uint16_t*)lora_b, r, lora_scale,
                      (const uint16_t*)residual, M, N);
   return check_launch();
+}
+
+extern "C" int tmx_qlora_gate_up_swiglu(void* stream, const void* x, const void* qweight, const void* scales,
+                                        const void* lora_a_t, const void* lora_b, void* act, int M, int K,
+                                        int F, int G, int r, float lora_scale) {
+  return qlinear_gate_up_swiglu((hipStream_t)stream, x, K, qweight, scales, lora_a_t, lora_b, r, lora_scale, act,
+                                M, K, F, G);
 }

@@ -66,6 +66,65 @@ __device__ __forceinline__ int acc_row(int r, int lane) {
   return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
 }
 
+// Expand one 32-bit word (8 nibbles, element j = 2 (i % 4) + i / 4 for nibble i)
+// into the 8 bf16 B-operand values of one MFMA step: bf16((u - 8) * s).
+__device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s) {
+  uint32_t lo = d & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
+  uint32_t hi = (d >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7 in bytes 0..3
+  // keep the two masked words opaque so that each byte is widened by one
+  // v_cvt_f32_ubyteN instead of a bit-field extract plus a conversion
+  asm volatile("" : "+v"(lo), "+v"(hi));
+  // nibble i: byte i/2 of (i even ? lo : hi)
+  const float n0 = (float)(lo & 0xFF), n1 = (float)(hi & 0xFF);
+  const float n2 = (float)((lo >> 8) & 0xFF), n3 = (float)((hi >> 8) & 0xFF);
+  const float n4 = (float)((lo >> 16) & 0xFF), n5 = (float)((hi >> 16) & 0xFF);
+  const float n6 = (float)(lo >> 24), n7 = (float)(hi >> 24);
+  // register p holds elements j = 2p, 2p + 1  <->  nibbles p, p + 4
+  uint32_t p[4];
+  p[0] = pack_bf2(fmaf(n0, s, m8s), fmaf(n4, s, m8s));
+  p[1] = pack_bf2(fmaf(n1, s, m8s), fmaf(n5, s, m8s));
+  p[2] = pack_bf2(fmaf(n2, s, m8s), fmaf(n6, s, m8s));
+  p[3] = pack_bf2(fmaf(n3, s, m8s), fmaf(n7, s, m8s));
+  bf16x8_t b;
+  __builtin_memcpy(&b, p, 16);
+  return b;
+}
+
+
+template <int V>
+struct IC { static constexpr int value = V; };
+
+// f(IC<0>{}), ..., f(IC<N - 1>{}): a loop whose index is a compile-time constant
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(IC<I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
+// Raw buffer descriptor over `bytes` bytes at p (loads take a per-lane and a scalar byte offset).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// 1 KiB from global memory straight into LDS (buffer_load ... lds): lane i's 16 bytes at byte
+// offset voffset + soffset of the buffer land at dst + 16 i; dst and soffset are wave-uniform.
+// Counted by vmcnt like any other load.
+__device__ __forceinline__ void load_row_to_lds(__amdgpu_buffer_rsrc_t r, void* dst, int voffset, int soffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16, voffset, soffset, 0, 0);
+}
+
+// Clock stamps per wave for profiling builds (TMX_PROF_STAMPS defined); nothing otherwise.
+#ifdef TMX_PROF_STAMPS
+__device__ unsigned long long* g_stamps;  // [workgroup][wave][32]
+#define TMX_STAMP(i)                                                                              \
+  if (g_stamps && lane == 0)                                                                      \
+  g_stamps[((size_t)blockIdx.x * (blockDim.x >> 6) + wave) * 32 + (i)] = wall_clock64()
+#else
+#define TMX_STAMP(i)
+#endif
+
 inline int check_launch() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TMX_OK : TMX_ERR_LAUNCH;
