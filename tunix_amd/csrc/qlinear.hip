@@ -648,7 +648,7 @@ struct GU8 {
   static constexpr int XS = TS * 64 + 8;       // bf16 elements per LDS row
   static constexpr int ROWS = MT * 32;
   static constexpr size_t SLAB = (size_t)2 * ROWS * XS * 2;
-  static constexpr size_t EPI = (size_t)8 * MT * 16 * 64 * 4 + (size_t)ROWS * 40 * 2;
+  static constexpr size_t EPI = (size_t)12 * MT * 16 * 64 * 4 + (size_t)ROWS * 40 * 2;
   static constexpr size_t LDS = SLAB > EPI ? SLAB : EPI;
 };
 
@@ -674,6 +674,16 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   const int wv = (nb * KT * 64 + lane) * 16;  // per-lane byte offsets
   const int sv = (nb * KG * 32 + nl) * 2;
   const int lv = lane * 64;
+  // LoRA B values of this tile's columns for the epilogue (rows h * 8 .. + 7 of B): read now, so
+  // that the cold reads complete under the main loop
+  uint16_t tbv[8];
+  if constexpr (FUSE) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = h * 8 + j;
+      tbv[j] = a.lora_b[(size_t)(k < a.lora_r ? k : 0) * a.N + nb * 32 + nl];
+    }
+  }
 
   f32x16_t acc[MT], tacc[FUSE ? MT : 1];
 #pragma unroll
@@ -770,17 +780,16 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     __syncthreads();
   };
 
+  // first step's operands, then (behind the first barrier's wait) the second step's weights
   dma_x(0, 0);
   static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(0, IC<0>{}, jc); });
-  static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(1, IC<1>{}, jc); });
-  if constexpr (FUSE) {
-    load_l(0, IC<0>{});
-    load_l(1, IC<1>{});
-  }
+  if constexpr (FUSE) load_l(0, IC<0>{});
   TMX_STAMP(1);
   __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_waitcnt(0x0F70 | ((TPW * 4 + (FUSE ? 8 : 0)) & 15) | (((TPW * 4 + (FUSE ? 8 : 0)) >> 4) << 14));
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
   __syncthreads();
+  static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(1, IC<1>{}, jc); });
+  if constexpr (FUSE) load_l(1, IC<1>{});
   TMX_STAMP(2);
   const int npairs = nsteps / 2;
   for (int g = 0; g < npairs; ++g) {
@@ -793,38 +802,39 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   TMX_STAMP(29);
 
   // ---- epilogue (the slab is free: the last step ended with a barrier) ----
+  // LDS regions (f32 unless noted): P [8 waves][MT][16][64] partial LoRA tiles, later reused as
+  // Y [4 tiles][MT][16][64] finished gate / up values; H [4 tiles][MT][16][64] accumulators of the
+  // second k-half; ts bf16 [ROWS][40] the LoRA projection t
   float* fl = reinterpret_cast<float*>(smem);
-  f32x16_t dl[MT];
-#pragma unroll
-  for (int m = 0; m < MT; ++m)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dl[m][r] = 0.f;
+  float* hb = fl + 8 * MT * 1024;
+  uint16_t* ts = reinterpret_cast<uint16_t*>(fl + 12 * MT * 1024);
+  bf16x8_t tb;
   if constexpr (FUSE) {
-    // B fragment of this tile's columns (rows beyond the rank are zero, which also masks the t
-    // columns of the other projection inside the 16-wide k window); fetched before the barriers
-    // below so that the cold reads overlap them
-    bf16x8_t tb;
-    {
-      const int colw = nb * 32 + nl;
-      float bv[8];
+    // B fragment of this tile's columns: rows beyond the rank are zero, which also masks the t
+    // columns of the other projection inside the 16-wide k window
+    uint16_t bz[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int k = h * 8 + j;
-        bv[j] = k < a.lora_r ? bf2f(a.lora_b[(size_t)k * a.N + colw]) : 0.f;
-      }
-      uint32_t pb[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) pb[j] = pack_bf2(bv[2 * j], bv[2 * j + 1]);
-      __builtin_memcpy(&tb, pb, 16);
-    }
-    // 1. t = x . [A_gate | A_up]: the partial tiles of all waves meet in LDS, are summed in wave
-    // order, rounded to bf16 and laid out row-major for the MFMA A fragments of step 2
-    uint16_t* ts = reinterpret_cast<uint16_t*>(fl + 8 * MT * 16 * 64);  // [ROWS][40]
+    for (int j = 0; j < 8; ++j) bz[j] = (h * 8 + j) < a.lora_r ? tbv[j] : (uint16_t)0;
+    __builtin_memcpy(&tb, bz, 16);
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int r = 0; r < 16; ++r) fl[(((wave * MT + m) * 16 + r) << 6) + lane] = tacc[m][r];
-    __syncthreads();
+  }
+  // the two k-halves of a tile swap halves of their accumulators: the first half finishes
+  // registers 0..7, the second 8..15 (a + b == b + a: the sum does not depend on who adds)
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r8 = 0; r8 < 8; ++r8) {
+      const int r = kh ? r8 : r8 + 8;
+      hb[(((cw * MT + m) * 16 + r) << 6) + lane] = kh ? acc[m][r8] : acc[m][r8 + 8];
+    }
+  TMX_STAMP(20);
+  __syncthreads();
+  TMX_STAMP(21);
+  if constexpr (FUSE) {
+    // t = x . [A_gate | A_up]: partial tiles summed in wave order, rounded to bf16, row-major
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -835,58 +845,52 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
         for (int w = 0; w < 8; ++w) t += fl[(((w * MT + m) * 16 + r) << 6) + lane];
         ts[(m * 32 + acc_row(r, lane)) * 40 + nl] = f2bf(t);
       }
+    TMX_STAMP(22);
     __syncthreads();
-    if (kh == 0) {
-      // 2. delta = t . B on the MFMA
-      const int toff = (cw >= 2) ? a.lora_r : 0;
+    TMX_STAMP(23);
+  }
+  {
+    // y = bf16(x . W) (+ bf16(bf16(t . B) * ls)): the LoRA product runs on the MFMA, t rows as A
+    // fragments, the B columns of this tile as B fragments, k = rank padded with zeros
+    const int toff = (cw >= 2) ? a.lora_r : 0;
 #pragma unroll
-      for (int m = 0; m < MT; ++m) {
+    for (int m = 0; m < MT; ++m) {
+      f32x16_t dl;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dl[r] = 0.f;
+      if constexpr (FUSE) {
         uint16_t tv[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) tv[j] = ts[(m * 32 + nl) * 40 + toff + h * 8 + j];
         bf16x8_t ta;
         __builtin_memcpy(&ta, tv, 16);
-        dl[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta, tb, dl[m], 0, 0, 0);
+        dl = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta, tb, dl, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r8 = 0; r8 < 8; ++r8) {
+        const int r = kh ? r8 + 8 : r8;
+        float y = rbf((kh ? acc[m][r8 + 8] : acc[m][r8]) + hb[(((cw * MT + m) * 16 + r) << 6) + lane]);
+        if (FUSE) y = rbf(y + rbf(rbf(kh ? dl[r8 + 8] : dl[r8]) * a.lora_ls));
+        fl[(((cw * MT + m) * 16 + r) << 6) + lane] = y;  // partial tiles were consumed before the last barrier
       }
     }
-    __syncthreads();  // ts / partial tiles are overwritten below
   }
-  // the second k-half hands its accumulators to the first
-  if (kh == 1) {
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) fl[(((cw * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
-  }
+  TMX_STAMP(24);
   __syncthreads();
-  if (kh == 0) {
+  TMX_STAMP(25);
+  // act = bf16(bf16(g * bf16(sigmoid(g))) * u): every wave finishes a quarter of one gate tile
+  {
+    const int gt = wave & 1, q = wave >> 1;
+    const int col = ((int)blockIdx.x * 2 + gt) * 32 + nl;
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float y = rbf(acc[m][r] + fl[(((cw * MT + m) * 16 + r) << 6) + lane]);
-        if (FUSE) y = rbf(y + rbf(rbf(dl[m][r]) * a.lora_ls));
-        acc[m][r] = y;
-      }
-  }
-  __syncthreads();
-  // act = bf16(bf16(g * bf16(sigmoid(g))) * u): the up waves hand their tile to the gate waves
-  if (kh == 0 && cw >= 2) {
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) fl[((((cw - 2) * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
-  }
-  __syncthreads();
-  if (kh == 0 && cw < 2) {
-    const int col = ((int)blockIdx.x * 2 + cw) * 32 + nl;
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int rr = 0; rr < 4; ++rr) {
+        const int r = q * 4 + rr;
         const int row = m * 32 + acc_row(r, lane);
         if (row >= a.M) continue;
-        const float g = acc[m][r], u = fl[(((cw * MT + m) * 16 + r) << 6) + lane];
+        const float g = fl[(((gt * MT + m) * 16 + r) << 6) + lane];
+        const float u = fl[((((2 + gt) * MT + m) * 16 + r) << 6) + lane];
         const float sg = rbf(1.f / (1.f + expf(-g)));
         a.y_bf16[(size_t)row * a.ldy + col] = f2bf(rbf(g * sg) * u);
       }
