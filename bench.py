@@ -291,8 +291,16 @@ def main():
       else:
         dense.append(('gate_up_linear', 'gate_up'))
       dense.append(('down_linear', 'down'))
+    def kway_symbol(pl):
+      # slices of whole 8-tile steps (up to 64 rows) run the direct-to-LDS variant of the k-way kernel
+      ns = lib.tmx_qlora_linear_num_splits(batch, pl.k, pl.n)
+      kt = pl.k // 64
+      slice_len = ((kt + ns - 1) // ns + 3) // 4 * 4
+      if batch <= 64 and pl.k % 512 == 0 and slice_len % 8 == 0:
+        return f'tmx::qlinear_mfma_dma_kernel<{mt}>'
+      return f'tmx::qlinear_mfma_kernel<{mt}, 2>'
     for cls_name, key in dense:
-      sym = f'tmx::qlinear_mfma4_kernel<{mt}>' if four(layer0[key]) else f'tmx::qlinear_mfma_kernel<{mt}, 2>'
+      sym = f'tmx::qlinear_mfma4_kernel<{mt}>' if four(layer0[key]) else kway_symbol(layer0[key])
       symbols.setdefault(sym, []).append(cls_name)
     symbols.update({
         f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention'],

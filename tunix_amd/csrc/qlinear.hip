@@ -909,6 +909,183 @@ static int launch_gate_up8(hipStream_t st, const QLinearArgs& a) {
   return check_launch();
 }
 
+// ---------------------------------------------------------------------------
+// The k-way block for slices made of whole steps (K % 512 == 0, slice lengths % 8 == 0, up to
+// 64 rows): same work split as gemm_block<MT, 2> (wave (ct, kw): column tile ct, k-tiles
+// kw * 4 .. kw * 4 + 3 of every 8-tile step), but every global read is a buffer load with a
+// fixed per-lane offset and a scalar offset that advances per step, and the activation slab
+// goes from global memory straight into LDS (one 1 KiB row per load), so the loop has no
+// per-lane address arithmetic, no staging registers and no LDS stores.
+struct KD {
+  static constexpr int TS = 8, TPW = 4, XS = TS * 64 + 8;
+  static constexpr size_t lds(int MT) { return (size_t)2 * MT * 32 * XS * 2; }
+};
+
+template <int MT, bool LORA>
+__device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* smem) {
+  constexpr int TS = KD::TS, TPW = KD::TPW, XS = KD::XS, ROWS = MT * 32;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), ct = wave & 3, kw = wave >> 2;
+  const int h = lane >> 5, nl = lane & 31;
+  const int KT = a.K >> 6;
+  const int slice = LORA ? ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y
+                         : (int)blockIdx.y;
+  const int per = LORA ? a.kt_per_lora_split : a.kt_per_split;
+  const int kb0 = slice * per;
+  const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
+  const int nsteps = (kb1 - kb0) / TS, last_step = nsteps - 1;  // host: whole steps
+  if (nsteps <= 0) return;
+  const int gs = __builtin_ctz(a.G >> 6), KG = a.K / a.G;
+  const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
+  const int nb = LORA ? ct : (int)blockIdx.x * 4 + ct;
+  const bool tile_ok = nb < NT;  // waves past the last tile only help with the slab
+
+  const __amdgpu_buffer_rsrc_t rw =
+      LORA ? make_rsrc(a.a_t, (uint32_t)KT * NT * 4096u) : make_rsrc(a.qw, (uint32_t)NT * KT * 1024u);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scales, LORA ? 0u : (uint32_t)NT * KG * 64u);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, (uint32_t)a.M * a.ldx * 2u);
+  // LoRA: A in fragment order [K/64][NT][64 lanes][4][8], 4 KiB per (k-tile, column tile)
+  const int wv = LORA ? nb * 4096 + lane * 64 : (nb * KT * 64 + lane) * 16;
+  const int wstep = LORA ? NT * 4096 : 1024;  // bytes between consecutive k-tiles
+  const int sv = (nb * KG * 32 + nl) * 2;
+  const int xv = lane * 16;
+  constexpr int XR = ROWS / 8;  // slab rows per wave and step
+  int xrow_off[XR];
+#pragma unroll
+  for (int i = 0; i < XR; ++i) {
+    const int row_l = wave + 8 * i;
+    xrow_off[i] = (row_l < a.M ? row_l : a.M - 1) * a.ldx * 2 + kb0 * 128;
+  }
+
+  f32x16_t acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
+  constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
+  constexpr int DW = LORA ? 1 : 2;   // steps of weights in flight
+  u32x4_t wring[DW][TPW][WPT];
+  uint16_t sring[DW][TPW];
+
+  auto load_w_tile = [&](int step, auto dc, auto jc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+    step = step < last_step ? step : last_step;
+    const int kt = kb0 + step * TS + kw * TPW + j;
+#pragma unroll
+    for (int t = 0; t < WPT; ++t) wring[d][j][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv + t * 16, kt * wstep, 0);
+    if (!LORA) sring[d][j] = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
+  };
+  auto dma_x = [&](int step, int buf) __attribute__((always_inline)) {
+    step = step < last_step ? step : last_step;
+    uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * XS;
+#pragma unroll
+    for (int i = 0; i < XR; ++i) load_row_to_lds(rx, base + i * 8 * XS, xv, xrow_off[i] + step * (TS * 128));
+  };
+  auto tile_math = [&](int step, int buf, auto dc, auto jc) __attribute__((always_inline)) {
+    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kw * TPW + j) * 64 + h * 8 + nl * XS;
+    bf16x8_t xa[MT][4];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + t * 16);
+    u32x4_t wc[WPT];
+#pragma unroll
+    for (int t = 0; t < WPT; ++t) wc[t] = wring[d][j][t];
+    const float s_c = LORA ? 0.f : bf2f(sring[d][j]);
+    load_w_tile(step + DW, dc, jc);  // slot consumed: refill it DW steps ahead
+    const float m8s = -8.f * s_c;
+    const uint32_t wd[4] = {wc[0].x, wc[0].y, wc[0].z, wc[0].w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      bf16x8_t b;
+      if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[t % WPT]);
+      else b = dequant_word(wd[t], s_c, m8s);
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[m], 0, 0, 0);
+    }
+  };
+  // loads of a step younger than its slab transfer (in-order counter: waiting until only these
+  // are outstanding completes the slab while the weight prefetch stays in flight)
+  constexpr int kYounger = TPW * (LORA ? 4 : 2);
+  auto wait_slab = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    if (tile_ok) __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  };
+  auto do_step = [&](int step, auto sc) __attribute__((always_inline)) {
+    constexpr int sp = decltype(sc)::value;
+    constexpr int d = sp % DW;
+    dma_x(step + 1, sp ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (tile_ok)
+      static_for<TPW>([&](auto jc) __attribute__((always_inline)) { tile_math(step, sp, IC<d>{}, jc); });
+    wait_slab();
+  };
+
+  dma_x(0, 0);
+  if (tile_ok) static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(0, IC<0>{}, jc); });
+  wait_slab();
+  if (DW == 2 && tile_ok)
+    static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(1, IC<1 % DW>{}, jc); });
+  const int npairs = nsteps / 2;
+  for (int g = 0; g < npairs; ++g) {
+    do_step(2 * g, IC<0>{});
+    do_step(2 * g + 1, IC<1>{});
+  }
+  if (nsteps & 1) do_step(nsteps - 1, IC<0>{});
+
+  // the two k-halves of a tile swap halves of their accumulators through LDS (the slab is free:
+  // the last step ended with a barrier): the first finishes registers 0..7, the second 8..15
+  float* hb = reinterpret_cast<float*>(smem);  // [4 tiles][MT][16][64]
+  if (tile_ok) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r8 = 0; r8 < 8; ++r8) {
+        const int r = kw ? r8 : r8 + 8;
+        hb[(((ct * MT + m) * 16 + r) << 6) + lane] = kw ? acc[m][r8] : acc[m][r8 + 8];
+      }
+  }
+  __syncthreads();
+  if (!tile_ok) return;
+  const int col = nb * 32 + nl;
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r8 = 0; r8 < 8; ++r8) {
+      const int r = kw ? r8 + 8 : r8;
+      const int row = m * 32 + acc_row(r, lane);
+      if (row >= a.M) continue;
+      const float mine = kw ? acc[m][r8 + 8] : acc[m][r8], other = hb[(((ct * MT + m) * 16 + r) << 6) + lane];
+      const float v = kw ? other + mine : mine + other;  // first half + second half
+      if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = v;
+      else if (a.y_bf16) a.y_bf16[(size_t)row * a.ldy + col] = f2bf(v);
+      else a.y_part[((size_t)slice * a.M + row) * a.N + col] = v;
+    }
+}
+
+template <int MT>
+__global__ __launch_bounds__(512, 1) void qlinear_mfma_dma_kernel(QLinearArgs a) {
+  extern __shared__ __align__(16) uint16_t smem[];
+  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block_dma<MT, true>(a, smem);
+  else gemm_block_dma<MT, false>(a, smem);
+}
+
+template <int MT>
+static int launch_qlinear_dma(hipStream_t st, QLinearArgs a) {
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&qlinear_mfma_dma_kernel<MT>), hipFuncAttributeMaxDynamicSharedMemorySize,
+      (int)KD::lds(MT));
+  if (attr != hipSuccess) return TMX_ERR_LAUNCH;
+  a.n_main_blocks = (a.N + 127) / 128;
+  const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
+  hipLaunchKernelGGL((qlinear_mfma_dma_kernel<MT>), dim3(blocks, a.nsplit), dim3(512), KD::lds(MT), st, a);
+  return check_launch();
+}
+
 // Which kernel serves a projection: the 4-wave kernel needs K % 256 == 0; deep projections
 // (K >= 8192) and mid-width ones (40 to 191 column blocks: enough workgroups of 8 waves to fill
 // the CUs in one round; measured on the q|k|v shape) go to the k-way kernel.
@@ -1058,6 +1235,10 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
     if (M <= 64) return launch_qlinear4<2>(st, a);
     return launch_qlinear4<4>(st, a);
   }
+  // slices of whole 8-tile steps, up to 64 rows, 32-bit byte offsets: the direct-to-LDS variant
+  if (M <= 64 && K % 512 == 0 && a.kt_per_split % 8 == 0 && (!a_t || a.kt_per_lora_split % 8 == 0) &&
+      (size_t)M * ldx * 2 < (1u << 31) && (size_t)K * N / 2 < (1u << 31) && (size_t)K * Rpad * 2 < (1u << 31))
+    return M <= 32 ? launch_qlinear_dma<1>(st, a) : launch_qlinear_dma<2>(st, a);
   if (M <= 32) return launch_qlinear<1, 2>(st, a);
   if (M <= 64) return launch_qlinear<2, 2>(st, a);
   return launch_qlinear<4, 2>(st, a);
