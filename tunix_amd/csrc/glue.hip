@@ -88,6 +88,26 @@ __device__ __forceinline__ void stage_t(float* t_s, const LoraIn& l, int m, int 
                                            (size_t)M * l.ldt, l.nsplit));
 }
 
+// The same for a whole workgroup: every (plane, column) value is fetched by its own thread
+// (one memory latency instead of one per batch of planes), parked in `stage`
+// [nsplit][n] floats, then the first n threads add their column's planes in ascending order.
+// Ends with a barrier; needs n * nsplit <= the capacity of `stage`.
+__device__ __forceinline__ void stage_t_block(float* t_s, float* stage, const LoraIn& l, int m, int M, int col0,
+                                              int n) {
+  const int total = n * l.nsplit;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    const int sp = i / n, c = i - sp * n;
+    stage[i] = l.t_part[((size_t)sp * M + m) * l.ldt + col0 + c];
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < n) {
+    float t = 0.f;
+    for (int sp = 0; sp < l.nsplit; ++sp) t += stage[sp * n + threadIdx.x];
+    t_s[threadIdx.x] = rbf(t);
+  }
+  __syncthreads();
+}
+
 // 8 adjacent outputs n0..n0+7 of one row: base = bf16(sum of the split planes) or the bf16 tensor.
 __device__ __forceinline__ void load_base8(const uint16_t* y_bf16, const float* y_part, int nsplit, int m,
                                            int M, int N, int n0, float* o) {
@@ -104,13 +124,24 @@ __device__ __forceinline__ void load_base8(const uint16_t* y_bf16, const float* 
     case 8: sum_planes8<8>(p, stride, o); break;
     case 16: sum_planes8<16>(p, stride, o); break;
     default: {
+      // any other count: up to 16 planes in flight at once (clamped, in-bounds plane indices),
+      // added in ascending order like the fixed counts
 #pragma unroll
       for (int e = 0; e < 8; ++e) o[e] = 0.f;
-      for (int s = 0; s < nsplit; ++s) {
-        float t[8];
-        sum_planes8<1>(p + (size_t)s * stride, stride, t);
+      for (int s0 = 0; s0 < nsplit; s0 += 16) {
+        float4 a[16], b[16];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] += t[e];
+        for (int i = 0; i < 16; ++i) {
+          const float4* q = reinterpret_cast<const float4*>(p + (size_t)(s0 + i < nsplit ? s0 + i : nsplit - 1) * stride);
+          a[i] = q[0];
+          b[i] = q[1];
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (s0 + i < nsplit) {
+            o[0] += a[i].x; o[1] += a[i].y; o[2] += a[i].z; o[3] += a[i].w;
+            o[4] += b[i].x; o[5] += b[i].y; o[6] += b[i].z; o[7] += b[i].w;
+          }
       }
     }
   }
@@ -140,6 +171,7 @@ template <int CPT>  // 8-element chunks per thread, D <= 4096 * CPT
 __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
   __shared__ float smem[8];
   __shared__ float t_s[TMX_MAX_RPAD];
+  __shared__ float t_stage[TMX_MAX_LORA_SPLITS * 64];
   const int m = blockIdx.x, M = gridDim.x;
   float v[CPT][8];
   float ss = 0.f;
@@ -188,9 +220,33 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
       }
     }
   }
-  if (!src && a.lora.t_part) {
-    stage_t(t_s, a.lora, m, M, 0, a.lora.r);
-    __syncthreads();
+  // rows of B for this thread's columns and the norm weights: requested now, used after the
+  // barriers below (one row = 16 bytes per thread; up to 16 rows are kept in registers when
+  // every thread owns a single chunk)
+  constexpr int kBR = CPT == 1 ? 16 : 1;
+  const bool lora = !src && a.lora.t_part;
+  const bool b_early = CPT == 1 && lora && a.lora.r <= kBR && (int)threadIdx.x < nchunks;
+  uint4 brow[kBR];
+  if (b_early) {
+#pragma unroll
+    for (int rr = 0; rr < kBR; ++rr)
+      brow[rr] = *reinterpret_cast<const uint4*>(a.lora.b + (size_t)(rr < a.lora.r ? rr : 0) * a.D + threadIdx.x * 8);
+  }
+  uint4 nw4[CPT];
+  if (a.norm_w) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int c = threadIdx.x + 512 * i;
+      nw4[i] = *reinterpret_cast<const uint4*>(a.norm_w + (c < nchunks ? c : 0) * 8);
+    }
+  }
+  if (lora) {
+    if (a.lora.r * a.lora.nsplit <= TMX_MAX_LORA_SPLITS * 64) {
+      stage_t_block(t_s, t_stage, a.lora, m, M, 0, a.lora.r);
+    } else {
+      stage_t(t_s, a.lora, m, M, 0, a.lora.r);
+      __syncthreads();
+    }
   }
 #pragma unroll
   for (int i = 0; i < CPT; ++i) {
@@ -198,7 +254,21 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
     if (c < nchunks) {
       const int n0 = c * 8;
       if (!src) {
-        if (a.lora.t_part) add_lora8(v[i], t_s, a.lora.b, a.D, n0, a.lora.r, a.lora.ls);
+        if (b_early) {
+          float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int rr = 0; rr < kBR; ++rr) {
+            float wv[8];
+            unpack8(brow[rr], wv);
+            const float t = rr < a.lora.r ? t_s[rr] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) d[e] = fmaf(t, wv[e], d[e]);
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e] + rbf(rbf(d[e]) * a.lora.ls));
+        } else if (lora) {
+          add_lora8(v[i], t_s, a.lora.b, a.D, n0, a.lora.r, a.lora.ls);
+        }
         if (a.residual) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e] + res8[i][e]);
@@ -218,7 +288,7 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
     if (c < nchunks) {
       const int n0 = c * 8;
       float w[8], o[8];
-      unpack8(*reinterpret_cast<const uint4*>(a.norm_w + n0), w);
+      unpack8(nw4[i], w);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         if (a.family == TMX_FAMILY_LLAMA3) o[e] = rbf(w[e] * v[i][e]) / rms;
