@@ -640,7 +640,9 @@ static int launch_qlinear(hipStream_t st, QLinearArgs a) {
 // column tile: wave (cw, kh) multiplies tile cw by k-tiles kh * TPW .. kh * TPW + TPW - 1 of
 // every step (starting at k-tile kh * TPW + cw, the one whose LoRA product x . A it also owns), so each SIMD holds two waves whose dequantisation, MFMA and load waits overlap.
 // All global reads are buffer loads: a per-lane byte offset that never changes plus a scalar
-// offset that advances per step, so the loop carries no per-lane address arithmetic.
+// offset that advances per step, so the loop carries no per-lane address arithmetic.  Weights
+// are requested one step (3-4 us) ahead: a deeper ring only lengthened the queue in front of the
+// memory pipeline (measured).
 template <int MT>
 struct GU8 {
   static constexpr int TS = 8;                 // k-tiles per step
@@ -707,16 +709,16 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     const int row_l = wave + 8 * i;
     xrow_off[i] = (row_l < a.M ? row_l : a.M - 1) * a.ldx * 2;
   }
-  u32x4_t wring[2][TPW];
-  uint16_t sring[2][TPW];
-  u32x4_t lring[FUSE ? 2 : 1][4];
+  u32x4_t wring[TPW];   // weights of the next step (refilled tile by tile as they are consumed)
+  uint16_t sring[TPW];
+  u32x4_t lring[4];
 
-  auto load_w_tile = [&](int step, auto dc, auto jc) __attribute__((always_inline)) {
-    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+  auto load_w_tile = [&](int step, auto jc) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
     step = step < last_step ? step : last_step;
     const int kt = step * TS + kh * TPW + ((j + cw) & (TPW - 1));
-    wring[d][j] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv, kt * 1024, 0);
-    sring[d][j] = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
+    wring[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv, kt * 1024, 0);
+    sring[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
   };
   // global -> LDS without passing through registers (buffer_load ... lds: lane i lands at
   // base + 16 i, so a row of the slab arrives contiguously and the 16-byte row pad is skipped)
@@ -727,24 +729,23 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     for (int i = 0; i < XR; ++i)
       load_row_to_lds(rx, base + i * 8 * XS, xv, xrow_off[i] + step * (TS * 128));
   };
-  auto load_l = [&](int step, auto dc) __attribute__((always_inline)) {
-    constexpr int d = decltype(dc)::value;
+  auto load_l = [&](int step) __attribute__((always_inline)) {
     step = step < last_step ? step : last_step;
     const int so = (step * TS + kh * TPW + cw) * 4096;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) lring[d][t] = __builtin_amdgcn_raw_buffer_load_b128(rl, lv + t * 16, so, 0);
+    for (int t = 0; t < 4; ++t) lring[t] = __builtin_amdgcn_raw_buffer_load_b128(rl, lv + t * 16, so, 0);
   };
-  auto tile_math = [&](int step, int buf, auto dc, auto jc) __attribute__((always_inline)) {
-    constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
+  auto tile_math = [&](int step, int buf, auto jc) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
     const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kh * TPW + ((j + cw) & (TPW - 1))) * 64 + h * 8 + nl * XS;
     bf16x8_t xa[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int t = 0; t < 4; ++t) xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + t * 16);
-    const u32x4_t wc = wring[d][j];
-    const float s_c = bf2f(sring[d][j]);
-    load_w_tile(step + 2, dc, jc);  // slot consumed: refill it two steps ahead
+    const u32x4_t wc = wring[j];
+    const float s_c = bf2f(sring[j]);
+    load_w_tile(step + 1, jc);  // slot consumed: refill it for the next step
     const float m8s = -8.f * s_c;
     const uint32_t wd[4] = {wc.x, wc.y, wc.z, wc.w};
 #pragma unroll
@@ -757,12 +758,12 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     if constexpr (FUSE && j == 0) {  // the wave's first k-tile of a step is kh * TPW + cw: its LoRA share
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const bf16x8_t b = __builtin_bit_cast(bf16x8_t, lring[d][t]);
+        const bf16x8_t b = __builtin_bit_cast(bf16x8_t, lring[t]);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
           tacc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, tacc[m], 0, 0, 0);
       }
-      load_l(step + 2, dc);
+      load_l(step + 1);
     }
   };
   // Loads of a step younger than its slab transfer: a weight tile and a scale per k-tile plus the
@@ -774,22 +775,19 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     constexpr int sp = decltype(sc)::value;
     dma_x(step + 1, sp ^ 1);
     __builtin_amdgcn_sched_barrier(0);
-    static_for<TPW>([&](auto jc) __attribute__((always_inline)) { tile_math(step, sp, IC<sp>{}, jc); });
+    static_for<TPW>([&](auto jc) __attribute__((always_inline)) { tile_math(step, sp, jc); });
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
     __syncthreads();
   };
 
-  // first step's operands, then (behind the first barrier's wait) the second step's weights
   dma_x(0, 0);
-  static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(0, IC<0>{}, jc); });
-  if constexpr (FUSE) load_l(0, IC<0>{});
+  static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(0, jc); });
+  if constexpr (FUSE) load_l(0);
   TMX_STAMP(1);
   __builtin_amdgcn_sched_barrier(0);
   __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
   __syncthreads();
-  static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(1, IC<1>{}, jc); });
-  if constexpr (FUSE) load_l(1, IC<1>{});
   TMX_STAMP(2);
   const int npairs = nsteps / 2;
   for (int g = 0; g < npairs; ++g) {
@@ -963,7 +961,7 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
   constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
-  constexpr int DW = LORA ? 1 : 2;   // steps of weights in flight
+  constexpr int DW = 1;              // steps of weights in flight
   u32x4_t wring[DW][TPW][WPT];
   uint16_t sring[DW][TPW];
 
