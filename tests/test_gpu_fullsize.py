@@ -61,6 +61,54 @@ def test_projection_of_one_hot_rows_is_a_row_lookup(K, N, group):
                       min_exact=0.99, what=f'one-hot {K}x{N}')
 
 
+@pytest.mark.parametrize('M,r', [(64, 16), (64, 0), (17, 16)])
+def test_fused_gate_up_of_one_hot_rows_is_swiglu_of_a_row_lookup(M, r):
+  """gate | up + LoRA + SwiGLU in one launch at the 8B shape (K = 4096, F = 14336): with one-hot
+  activation rows the two projections are rows of the bit-exactly dequantised matrix, so the
+  activation is known in closed form."""
+  K, F, group = 4096, 14336, 64
+  g = torch.Generator(device=G.DEV).manual_seed(31 + M + r)
+  rnd = lambda *s: (torch.randn(*s, generator=g, device=G.DEV) * 0.05).to(torch.bfloat16)
+  ws = [rnd(K, F), rnd(K, F)]
+  loras = [(rnd(K, r), rnd(r, F)) for _ in range(2)] if r else None
+  pl = quant.PackedLinear.from_dense(ws, group, G.DEV, loras, 2.0)
+  dense = torch.empty(K, 2 * F, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_int4_dequant', S(), G.p(pl.qweight), G.p(pl.scales), G.p(dense), K, 2 * F, group)
+  ks = torch.randint(0, K, (M,), generator=g, device=G.DEV)
+  ks[0], ks[1], ks[2] = 0, K - 1, 511          # first / last row, step edge
+  amp = torch.full((M,), 8.0, device=G.DEV)     # |g| around 1: the sigmoid is exercised
+  amp[3], amp[4], amp[5] = -16.0, 0.5, 0.0
+  x = torch.zeros(M, K, dtype=torch.bfloat16, device=G.DEV)
+  x[torch.arange(M), ks] = amp.to(torch.bfloat16)
+  act = torch.empty(M, F, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_qlora_gate_up_swiglu', S(), G.p(x), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t), G.p(pl.lora_b),
+         G.p(act), M, K, F, group, r, 2.0)
+  G.sync()
+  y = _bf16_round(dense[ks].float() * amp[:, None])            # [M, 2F], exact
+  slack = torch.zeros_like(y)                                  # how far a last-bit flip of the LoRA sum can move y
+  if r:
+    for i, (a, b) in enumerate(loras):
+      t = _bf16_round(a[ks].float() * amp[:, None])
+      delta = _bf16_round(_bf16_round(t @ b.float()) * 2.0)
+      base = y[:, i * F:(i + 1) * F].clone()
+      y[:, i * F:(i + 1) * F] = _bf16_round(base + delta)
+      ulp = lambda v: torch.exp2(torch.floor(torch.log2(v.abs().clamp(min=2.0 ** -120))) - 7)
+      slack[:, i * F:(i + 1) * F] = torch.maximum(torch.maximum(ulp(base), ulp(delta)), ulp(y[:, i * F:(i + 1) * F]))
+  gte, up = y[:, :F], y[:, F:]
+  sg = _bf16_round(1.0 / (1.0 + torch.exp(-gte)))
+  want = _bf16_round(_bf16_round(gte * sg) * up)
+  if r == 0:
+    # no rounding freedom except the sigmoid's last bit (expf vs torch.exp)
+    G.assert_bf16_close(G.host(act), want.cpu().numpy(), ulps=1.0, min_exact=0.99, what='fused gate_up one-hot')
+  else:
+    # the r-term LoRA sum may round differently (f32 summation order): a last-bit flip of the delta
+    # moves g or u by `slack`, and the product by |d act / d g| <= 1.1 |u|, |d act / d u| = |silu(g)|
+    silu = (gte * sg).abs()
+    extra = 1.5 * (1.1 * slack[:, :F] * up.abs() + slack[:, F:] * silu).cpu().numpy()
+    G.assert_bf16_close(G.host(act), want.cpu().numpy(), ulps=2.0, extra=extra, min_exact=0.97,
+                        what='fused gate_up + LoRA one-hot')
+
+
 def test_attention_with_zero_query_is_the_mean_of_valid_values():
   B, N, Kh, H, C = 64, 32, 8, 128, 768
   g = torch.Generator(device=G.DEV).manual_seed(5)
