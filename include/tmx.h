@@ -64,9 +64,9 @@ int tmx_int4_dequant(void* stream, const void* qweight, const void* scales, void
 /* y[M, N] = bf16(x[M, K] . dequant(qweight)) (+ LoRA delta) (+ residual), M <= 128.
  * Replaces the qwix-wrapped Einsum / nnx.Linear call: tunix/models/llama3/model.py:216-218,
  * :489-496; tunix/models/qwen3/model.py:389-393, :1199-1208.
- *   lora_a_t : A in MFMA fragment order, bf16 [K/64][r_pad/32][64][4][8], r_pad % 32 == 0,
+ *   lora_a_t : A in MFMA fragment order, bf16 [K/64][r_pad/32][4][64][8], r_pad % 32 == 0,
  *              columns >= r zero (NULL: no LoRA): element A[64 kb + 16 t + 8 h + j][32 ct + c]
- *              at ((((kb * (r_pad/32) + ct) * 64 + 32 h + c) * 4 + t) * 8 + j)
+ *              at ((((kb * (r_pad/32) + ct) * 4 + t) * 64 + 32 h + c) * 8 + j)
  *   lora_b   : bf16 [r, N]
  *   residual : bf16 [M, N] or NULL; added after the LoRA delta, in bf16
  *   workspace: tmx_qlora_linear_workspace_bytes(M, K, N) bytes (f32 K-slice planes) */

@@ -33,7 +33,7 @@ constexpr int kXStride = kKS * 64 + 8;    // bf16 elements per LDS row
 
 // LORA = false: one int4 column tile per wave.  LORA = true: the block computes a K-slice
 // of t = x . A from bf16 tiles of A (one 32-column tile per wave); A is stored in MFMA
-// B-fragment order, [K/64][Rpad/32][64 lanes][4 steps][8], so a wave reads 4 KiB contiguously.
+// B-fragment order, [K/64][Rpad/32][4 steps][64 lanes][8]: each MFMA operand is one coalesced 1 KiB load.
 // FUSE = true (gate | up pairs with LoRA): every wave also multiplies one of the step's four
 // k-tiles by the 32-column tile of [A_gate | A_up], reusing the activation fragments it already
 // holds, so t = x . A is complete inside the workgroup when the epilogue needs it.
@@ -76,7 +76,7 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int r = 0; r < 16; ++r) tacc[m][r] = 0.f;
-    lsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + (size_t)lane * 4;  // Rpad == 32: 256 words per k-tile
+    lsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + lane;  // Rpad == 32: 256 words per k-tile, 64 per fragment
   }
 
   // cooperative activation load: chunk c = tid + 256 i -> row c / 32, 16-byte column c % 32
@@ -99,7 +99,7 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
   size_t wstep;  // 16-byte words between consecutive k-tiles of one column tile
   if (LORA) {
     wstep = (size_t)NT * 64 * 4;
-    wsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + ((size_t)nb * 64 + lane) * 4 + (size_t)kb0 * wstep;
+    wsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + (size_t)nb * 256 + lane + (size_t)kb0 * wstep;
   } else {
     wstep = 64;
     wsrc = reinterpret_cast<const u32x4_t*>(a.qw) + (size_t)nb * KT * 64 + lane + (size_t)kb0 * wstep;
@@ -117,7 +117,7 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
     step = step < last_step ? step : last_step;
     const int rel = step * kKS + kt;  // k-tile relative to kb0
 #pragma unroll
-    for (int t = 0; t < WPT; ++t) wring[d][kt][t] = wsrc[(size_t)rel * wstep + t];
+    for (int t = 0; t < WPT; ++t) wring[d][kt][t] = wsrc[(size_t)rel * wstep + t * (LORA ? 64 : 1)];
     if (!LORA) sring[d][kt] = ssrc[(size_t)((kb0 + rel) >> kpg_shift) * 32];
   };
   auto load_w = [&](int step, auto dc) __attribute__((always_inline)) {
@@ -140,7 +140,7 @@ __device__ __forceinline__ void gemm_block4(const QLinearArgs& a, uint16_t (*xs)
     step = step < last_step ? step : last_step;
     const size_t kb = (size_t)(kb0 + step * kKS + wave);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) lring[d][t] = lsrc[kb * 256 + t];
+    for (int t = 0; t < 4; ++t) lring[d][t] = lsrc[kb * 256 + t * 64];
   };
   // one of the four k-tiles of a step
   auto tile_math = [&](int step, int buf, auto dc, auto kc) __attribute__((always_inline)) {
@@ -433,7 +433,7 @@ struct Shape {
 };
 
 // LORA = false: int4 column tiles.  LORA = true: the block computes a K-slice of t = x . A from
-// bf16 tiles of A; A is stored in MFMA B-fragment order, [K/64][Rpad/32][64 lanes][4 steps][8],
+// bf16 tiles of A; A is stored in MFMA B-fragment order, [K/64][Rpad/32][4 steps][64 lanes][8],
 // so a wave reads the 4 KiB of a tile contiguously.
 template <int MT, int KW_, bool LORA>
 __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t* smem) {
@@ -488,7 +488,7 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t* smem)
   if (tile_ok) {
     if (LORA) {
       wstep = (size_t)NT * 64 * 4;
-      wsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + ((size_t)nb * 64 + lane) * 4 + (size_t)kb0 * wstep;
+      wsrc = reinterpret_cast<const u32x4_t*>(a.a_t) + (size_t)nb * 256 + lane + (size_t)kb0 * wstep;
     } else {
       wstep = 64;
       wsrc = reinterpret_cast<const u32x4_t*>(a.qw) + (size_t)nb * KT * 64 + lane + (size_t)kb0 * wstep;
@@ -508,7 +508,7 @@ __device__ __forceinline__ void gemm_block(const QLinearArgs& a, uint16_t* smem)
     int rel = step * KS + kw * TPW + j;  // k-tile relative to kb0
     rel = rel < last_tile ? rel : last_tile;
 #pragma unroll
-    for (int t = 0; t < WPT; ++t) wring[d][j][t] = wsrc[(size_t)rel * wstep + t];
+    for (int t = 0; t < WPT; ++t) wring[d][j][t] = wsrc[(size_t)rel * wstep + t * (LORA ? 64 : 1)];
     if (!LORA) sring[d][j] = ssrc[(size_t)((kb0 + rel) >> kpg_shift) * 32];
   };
   auto load_w = [&](int step, auto dc) __attribute__((always_inline)) {
@@ -675,7 +675,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   const __amdgpu_buffer_rsrc_t rl = make_rsrc(FUSE ? a.a_t : a.x, FUSE ? (uint32_t)KT * 4096u : 16u);
   const int wv = (nb * KT * 64 + lane) * 16;  // per-lane byte offsets
   const int sv = (nb * KG * 32 + nl) * 2;
-  const int lv = lane * 64;
+  const int lv = lane * 16;
   // LoRA B values of this tile's columns for the epilogue (rows h * 8 .. + 7 of B): read now, so
   // that the cold reads complete under the main loop
   uint16_t tbv[8];
@@ -733,7 +733,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     step = step < last_step ? step : last_step;
     const int so = (step * TS + kh * TPW + cw) * 4096;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) lring[t] = __builtin_amdgcn_raw_buffer_load_b128(rl, lv + t * 16, so, 0);
+    for (int t = 0; t < 4; ++t) lring[t] = __builtin_amdgcn_raw_buffer_load_b128(rl, lv + t * 1024, so, 0);
   };
   auto tile_math = [&](int step, int buf, auto jc) __attribute__((always_inline)) {
     constexpr int j = decltype(jc)::value;
@@ -942,8 +942,8 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
       LORA ? make_rsrc(a.a_t, (uint32_t)KT * NT * 4096u) : make_rsrc(a.qw, (uint32_t)NT * KT * 1024u);
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scales, LORA ? 0u : (uint32_t)NT * KG * 64u);
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, (uint32_t)a.M * a.ldx * 2u);
-  // LoRA: A in fragment order [K/64][NT][64 lanes][4][8], 4 KiB per (k-tile, column tile)
-  const int wv = LORA ? nb * 4096 + lane * 64 : (nb * KT * 64 + lane) * 16;
+  // LoRA: A in fragment order [K/64][NT][4][64 lanes][8], 4 KiB per (k-tile, column tile)
+  const int wv = LORA ? nb * 4096 + lane * 16 : (nb * KT * 64 + lane) * 16;
   const int wstep = LORA ? NT * 4096 : 1024;  // bytes between consecutive k-tiles
   const int sv = (nb * KG * 32 + nl) * 2;
   const int xv = lane * 16;
@@ -970,7 +970,7 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
     step = step < last_step ? step : last_step;
     const int kt = kb0 + step * TS + kw * TPW + j;
 #pragma unroll
-    for (int t = 0; t < WPT; ++t) wring[d][j][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv + t * 16, kt * wstep, 0);
+    for (int t = 0; t < WPT; ++t) wring[d][j][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv + t * 1024, kt * wstep, 0);
     if (!LORA) sring[d][j] = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
   };
   auto dma_x = [&](int step, int buf) __attribute__((always_inline)) {

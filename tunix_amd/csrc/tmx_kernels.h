@@ -9,7 +9,7 @@ struct QLinearArgs {
   int ldx;
   const uint4* qw;         // packed int4 tiles
   const uint16_t* scales;  // [N/32][K/G][32] bf16
-  const uint16_t* a_t;     // LoRA A in fragment order [K/64][Rpad/32][64][4][8] bf16 (may be null)
+  const uint16_t* a_t;     // LoRA A in fragment order [K/64][Rpad/32][4][64][8] bf16 (may be null)
   uint16_t* y_bf16;        // [M, N] bf16 (only when nsplit == 1), else null
   float* y_part;           // [nsplit][M][N] f32 planes
   float* t_part;           // [lora splits][M][ldt] f32 LoRA projection planes

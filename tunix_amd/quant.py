@@ -51,16 +51,17 @@ def pad32(r):
 
 
 def pack_lora_a(a_list, k):
-  """[A_i [K, r]] -> bf16 [K // 64, r_pad // 32, 64, 4, 8]: the A matrices side by side,
+  """[A_i [K, r]] -> bf16 [K // 64, r_pad // 32, 4, 64, 8]: the A matrices side by side,
   zero-padded to a multiple of 32 columns, in MFMA B-fragment order: element
-  A[64 kb + 16 t + 8 h + j][32 ct + c] at [kb][ct][32 h + c][t][j]."""
+  A[64 kb + 16 t + 8 h + j][32 ct + c] at [kb][ct][t][32 h + c][j] (the operand of MFMA step
+  t of a tile is 1 KiB contiguous: lane 32 h + c reads 16 bytes at 16 * lane)."""
   a = torch.cat([x.to(torch.bfloat16) for x in a_list], dim=1)  # [K, R]
   r = a.shape[1]
   rp = pad32(r)
   full = torch.zeros(k, rp, dtype=torch.bfloat16, device=a.device)
   full[:, :r] = a
   t = full.reshape(k // 64, 4, 2, 8, rp // 32, 32)  # [kb, t, h, j, ct, c]
-  return t.permute(0, 4, 2, 5, 1, 3).reshape(k // 64, rp // 32, 64, 4, 8).contiguous()
+  return t.permute(0, 4, 1, 2, 5, 3).reshape(k // 64, rp // 32, 4, 64, 8).contiguous()
 
 
 class PackedLinear:
@@ -90,7 +91,7 @@ class PackedLinear:
   def lora_a_dense(self):
     """[K, r_pad] view of the packed A (inverse of pack_lora_a)."""
     kt, ct = self.lora_a_t.shape[0], self.lora_a_t.shape[1]
-    t = self.lora_a_t.reshape(kt, ct, 2, 32, 4, 8).permute(0, 4, 2, 5, 1, 3)  # [kb, t, h, j, ct, c]
+    t = self.lora_a_t.reshape(kt, ct, 4, 2, 32, 8).permute(0, 2, 3, 5, 1, 4)  # [kb, t, h, j, ct, c]
     return t.reshape(kt * 64, ct * 32)
 
   @classmethod
