@@ -37,6 +37,12 @@ static Splits plan_splits(const tmx_model_desc* m, int B) {
   s.qkv = qlinear_num_splits(D, QKV, B);
   s.o = qlinear_num_splits(NH, D, B);
   s.gate_up = m->num_experts > 0 ? 1 : qlinear_num_splits(D, 2 * F, B);
+  // up to 64 rows the 8-wave gate | up kernel (projection + LoRA + SwiGLU in one launch) beats a
+  // split projection plus a SwiGLU launch as soon as it has 64 workgroups to run
+  const tmx_qlinear_desc& gu = m->layers[0].gate_up;
+  if (m->num_experts == 0 && B <= 64 && D % 512 == 0 && D < 8192 && F % 64 == 0 && F / 64 >= 64 &&
+      (!gu.lora_a_t || (2 * gu.rank <= 32 && gu.r_pad == 32)))
+    s.gate_up = 1;
   s.down = m->num_experts > 0 ? 1 : qlinear_num_splits(F, D, B);
   return s;
 }
