@@ -98,8 +98,9 @@ def test_qlora_linear_planes_sum_and_rejects():
   assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, 129, K, N, group, 0, 1) == -2  # M > 128
   assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, M, K, N, 96, 0, 1) == -2      # G not a power of two
   assert lib.tmx_qlora_linear_planes(S(), 1, 1, 1, None, 1, None, M, K, N, group, 0, 3) == -2   # empty K-slice
-  assert lib.tmx_qlora_linear_num_lora_splits(4096, 4096) == 16 and lib.tmx_qlora_linear_num_lora_splits(14336, 4096) == 28
-  assert lib.tmx_qlora_linear_num_lora_splits(4096, 6144) == 8  # mid-width projection: 8-tile steps
+  # LoRA slices: whole groups of 4 k-tiles for narrow projections, of 8 from 16 column blocks on
+  assert lib.tmx_qlora_linear_num_lora_splits(4096, 1024) == 16 and lib.tmx_qlora_linear_num_lora_splits(14336, 4096) == 28
+  assert lib.tmx_qlora_linear_num_lora_splits(4096, 6144) == 8 and lib.tmx_qlora_linear_num_lora_splits(4096, 4096) == 8
 
 
 @pytest.mark.parametrize('family', [0, 1])

@@ -908,14 +908,17 @@ static int launch_gate_up8(hipStream_t st, const QLinearArgs& a) {
 }
 
 // ---------------------------------------------------------------------------
-// The k-way block for slices made of whole steps (K % 512 == 0, slice lengths % 8 == 0, up to
-// 64 rows): same work split as gemm_block<MT, 2> (wave (ct, kw): column tile ct, k-tiles
-// kw * 4 .. kw * 4 + 3 of every 8-tile step), but every global read is a buffer load with a
-// fixed per-lane offset and a scalar offset that advances per step, and the activation slab
-// goes from global memory straight into LDS (one 1 KiB row per load), so the loop has no
-// per-lane address arithmetic, no staging registers and no LDS stores.
+// The k-way block for slices made of whole 4-tile steps (K % 256 == 0, up to 64 rows): wave
+// (ct, kw) multiplies column tile ct by k-tiles 2 kw, 2 kw + 1 of every step.  Every global read
+// is a buffer load with a fixed per-lane offset and a scalar offset that advances per step, and
+// the activation slab goes from global memory straight into LDS, so the loop has no per-lane
+// address arithmetic, no staging registers and no LDS stores.  A slab row is 512 bytes; a
+// direct-to-LDS load lands 1 KiB contiguously, i.e. two rows back to back, so rows are stored
+// unpadded and the 16-byte chunks of row r are XOR-swizzled by r % 8 instead (the global
+// address of every lane is free, so the swizzle costs nothing; fragment reads stay
+// conflict-free).  64 KiB of LDS and <= 128 registers: two workgroups = 16 waves per CU.
 struct KD {
-  static constexpr int TS = 8, TPW = 4, XS = TS * 64 + 8;
+  static constexpr int TS = 4, TPW = 2, XS = 256;
   static constexpr size_t lds(int MT) { return (size_t)2 * MT * 32 * XS * 2; }
 };
 
@@ -946,13 +949,14 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
   const int wv = LORA ? nb * 4096 + lane * 16 : (nb * KT * 64 + lane) * 16;
   const int wstep = LORA ? NT * 4096 : 1024;  // bytes between consecutive k-tiles
   const int sv = (nb * KG * 32 + nl) * 2;
-  const int xv = lane * 16;
-  constexpr int XR = ROWS / 8;  // slab rows per wave and step
-  int xrow_off[XR];
+  // slab transfer: XR loads per wave and step; load i moves rows 2 wave + 16 i (lanes 0..31)
+  // and the next one (lanes 32..63), lane l delivering chunk (l % 32) ^ (row % 8) to slot l % 32
+  constexpr int XR = ROWS / 16;
+  int xoff[XR];  // per-lane byte offset of the row's first step (rows past M repeat the last)
 #pragma unroll
   for (int i = 0; i < XR; ++i) {
-    const int row_l = wave + 8 * i;
-    xrow_off[i] = (row_l < a.M ? row_l : a.M - 1) * a.ldx * 2 + kb0 * 128;
+    const int row_l = 2 * wave + 16 * i + h;
+    xoff[i] = (row_l < a.M ? row_l : a.M - 1) * a.ldx * 2 + ((nl ^ (row_l & 7)) * 16) + kb0 * 128;
   }
 
   f32x16_t acc[MT];
@@ -975,18 +979,21 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
   };
   auto dma_x = [&](int step, int buf) __attribute__((always_inline)) {
     step = step < last_step ? step : last_step;
-    uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * XS;
+    uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * 2 * XS;
 #pragma unroll
-    for (int i = 0; i < XR; ++i) load_row_to_lds(rx, base + i * 8 * XS, xv, xrow_off[i] + step * (TS * 128));
+    for (int i = 0; i < XR; ++i) load_row_to_lds(rx, base + i * 16 * XS, xoff[i], step * (TS * 128));
   };
   auto tile_math = [&](int step, int buf, auto dc, auto jc) __attribute__((always_inline)) {
     constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
-    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kw * TPW + j) * 64 + h * 8 + nl * XS;
+    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kw * TPW + j) * 64 + nl * XS;
     bf16x8_t xa[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + t * 16);
+      for (int t = 0; t < 4; ++t) {
+        // chunk 2 t + h of the tile sits at slot (2 t + h) ^ (row % 8)
+        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + (((2 * t + h) ^ (nl & 7)) * 8));
+      }
     u32x4_t wc[WPT];
 #pragma unroll
     for (int t = 0; t < WPT; ++t) wc[t] = wring[d][j][t];
@@ -1066,7 +1073,7 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
 }
 
 template <int MT>
-__global__ __launch_bounds__(512, 1) void qlinear_mfma_dma_kernel(QLinearArgs a) {
+__global__ __launch_bounds__(512, 2) void qlinear_mfma_dma_kernel(QLinearArgs a) {
   extern __shared__ __align__(16) uint16_t smem[];
   if ((int)blockIdx.x >= a.n_main_blocks) gemm_block_dma<MT, true>(a, smem);
   else gemm_block_dma<MT, false>(a, smem);
@@ -1085,12 +1092,15 @@ static int launch_qlinear_dma(hipStream_t st, QLinearArgs a) {
 }
 
 // Which kernel serves a projection: the 4-wave kernel needs K % 256 == 0; deep projections
-// (K >= 8192) and mid-width ones (40 to 191 column blocks: enough workgroups of 8 waves to fill
-// the CUs in one round; measured on the q|k|v shape) go to the k-way kernel.
+// (K >= 8192) and mid-width ones (enough column blocks to give every CU a workgroup of 8 waves
+// after the K split, fewer than the 192 from which a projection runs unsplit) go to the k-way
+// kernels.  Up to 64 rows the k-way kernel is the direct-to-LDS one, which wins from 16 column
+// blocks on (measured on the o shapes of the 8B and the 30B-A3B models and on q|k|v); above, from 40.
 static bool four_wave_shape(int K) { return K % 256 == 0 && K < 8192; }
-static bool four_wave(int K, int N) {
+static bool four_wave(int K, int N, int M) {
   const int nblocks = (N + 127) / 128;
-  return four_wave_shape(K) && !(nblocks >= 40 && nblocks < 192);
+  const int mid = M <= 64 ? 16 : 40;
+  return four_wave_shape(K) && !(nblocks >= mid && nblocks < 192);
 }
 
 static int slice_len(int KT, int s) { return ((KT + s - 1) / s + 3) / 4 * 4; }
@@ -1115,18 +1125,24 @@ static int num_splits4(int K, int N) {
   return best;
 }
 
+int qlinear_num_lora_splits(int K, int N);
 int qlinear_num_splits(int K, int N, int M) {
-  if (four_wave(K, N)) return num_splits4(K, N);
+  if (four_wave(K, N, M)) return num_splits4(K, N);
   const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
-  const int ks = M > 64 ? 4 : 8;
+  // steps of 4 k-tiles (direct-to-LDS kernel up to 64 rows, 128-row kernel) or 8; the workgroups
+  // of the LoRA projection share the launch, and a launch that does not fit one workgroup per CU
+  // pays a second round (measured: 272 workgroups run slower than 144 with twice the steps); the
+  // charge per plane covers the consumer's reads (measured on the o projection: 4 slices beat 6)
+  const int ks = (M > 64 || K % 256 == 0) ? 4 : 8;
+  const int nls = qlinear_num_lora_splits(K, N);
   int best = 1;
   float best_cost = 1e30f;
   for (int s = 1; s <= TMX_MAX_SPLITS; ++s) {
     if (!slices_ok(KT, s)) continue;
-    const int rounds = (nblocks * s + 255) / 256;
+    const int rounds = (nblocks * s + (nls + s - 1) / s * s + 255) / 256;
     const int nsteps = (slice_len(KT, s) + ks - 1) / ks;
-    const float cost = rounds * (nsteps + 2.0f) + 0.15f * s;
+    const float cost = rounds * (nsteps + (ks == 4 ? 4.0f : 2.0f)) + (ks == 4 ? 0.6f : 0.15f) * s;
     if (cost < best_cost) { best_cost = cost; best = s; }
   }
   return best;
@@ -1135,7 +1151,9 @@ int qlinear_num_splits(int K, int N, int M) {
 // Number of K-slices of the LoRA projection t = x . A: as fine as whole steps (4 or 8 k-tiles,
 // by kernel) allow, at most TMX_MAX_LORA_SPLITS planes, so that no LoRA block outlasts the
 // main blocks.
-static int lora_step(int K, int N) { return four_wave(K, N) ? 4 : 8; }
+// (the plane count is part of the interface and does not depend on the row count: 8 wherever
+// some row count picks a k-way kernel; the 4-wave kernel takes any multiple of 4)
+static int lora_step(int K, int N) { return four_wave(K, N, 1) ? 4 : 8; }
 int qlinear_num_lora_splits(int K, int N) {
   const int KT = K / 64, g = lora_step(K, N);
   for (int per = g;; per += g) {
@@ -1228,13 +1246,13 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   const int nls = qlinear_num_lora_splits(K, N);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
   a.kt_per_lora_split = lora_slice_len(K, N);
-  if (four_wave(K, N)) {
+  if (four_wave(K, N, M)) {
     if (M <= 32) return launch_qlinear4<1>(st, a);
     if (M <= 64) return launch_qlinear4<2>(st, a);
     return launch_qlinear4<4>(st, a);
   }
-  // slices of whole 8-tile steps, up to 64 rows, 32-bit byte offsets: the direct-to-LDS variant
-  if (M <= 64 && K % 512 == 0 && a.kt_per_split % 8 == 0 && (!a_t || a.kt_per_lora_split % 8 == 0) &&
+  // slices of whole steps, up to 64 rows, 32-bit byte offsets: the direct-to-LDS variant
+  if (M <= 64 && K % 256 == 0 && a.kt_per_split % 4 == 0 && (!a_t || a.kt_per_lora_split % 4 == 0) &&
       (size_t)M * ldx * 2 < (1u << 31) && (size_t)K * N / 2 < (1u << 31) && (size_t)K * Rpad * 2 < (1u << 31))
     return M <= 32 ? launch_qlinear_dma<1>(st, a) : launch_qlinear_dma<2>(st, a);
   if (M <= 32) return launch_qlinear<1, 2>(st, a);
