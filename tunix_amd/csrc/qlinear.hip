@@ -735,14 +735,20 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
 #pragma unroll
     for (int t = 0; t < 4; ++t) lring[t] = __builtin_amdgcn_raw_buffer_load_b128(rl, lv + t * 1024, so, 0);
   };
-  auto tile_math = [&](int step, int buf, auto jc) __attribute__((always_inline)) {
+  // activation fragments of the wave's j-th k-tile of a step, read one tile ahead of their use
+  bf16x8_t xq[2][MT][4];
+  auto read_x = [&](int buf, auto jc) __attribute__((always_inline)) {
     constexpr int j = decltype(jc)::value;
     const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kh * TPW + ((j + cw) & (TPW - 1))) * 64 + h * 8 + nl * XS;
-    bf16x8_t xa[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + t * 16);
+      for (int t = 0; t < 4; ++t) xq[j & 1][m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + t * 16);
+  };
+  auto tile_math = [&](int step, int buf, auto jc) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
+    if constexpr (j + 1 < TPW) read_x(buf, IC<j + 1>{});
+    auto& xa = xq[j & 1];
     const u32x4_t wc = wring[j];
     const float s_c = bf2f(sring[j]);
     load_w_tile(step + 1, jc);  // slot consumed: refill it for the next step
@@ -775,6 +781,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     constexpr int sp = decltype(sc)::value;
     dma_x(step + 1, sp ^ 1);
     __builtin_amdgcn_sched_barrier(0);
+    read_x(sp, IC<0>{});
     static_for<TPW>([&](auto jc) __attribute__((always_inline)) { tile_math(step, sp, jc); });
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
