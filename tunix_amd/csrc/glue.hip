@@ -190,7 +190,36 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
     }
   }
   const int nchunks = a.D >> 3;
-  // issue the row's own loads (planes, residual) before waiting on the staged LoRA vector
+  // Everything that does not depend on the row's own sums is requested first and in one go, so
+  // that the memory latencies overlap: the LoRA planes' values (one per thread), the rows of B
+  // for this thread's columns (16 bytes each; up to 16 rows are kept in registers when every
+  // thread owns a single chunk) and the norm weights.  The in-order load counter makes the wait
+  // for the planes below cover them all.
+  constexpr int kBR = CPT == 1 ? 16 : 1;
+  const bool lora = !src && a.lora.t_part;
+  const bool b_early = CPT == 1 && lora && a.lora.r <= kBR && (int)threadIdx.x < nchunks;
+  uint4 brow[kBR];
+  if (b_early) {
+#pragma unroll
+    for (int rr = 0; rr < kBR; ++rr)
+      brow[rr] = *reinterpret_cast<const uint4*>(a.lora.b + (size_t)(rr < a.lora.r ? rr : 0) * a.D + threadIdx.x * 8);
+  }
+  uint4 nw4[CPT];
+  if (a.norm_w) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int c = threadIdx.x + 512 * i;
+      nw4[i] = *reinterpret_cast<const uint4*>(a.norm_w + (c < nchunks ? c : 0) * 8);
+    }
+  }
+  const int t_total = lora ? a.lora.r * a.lora.nsplit : 0;
+  const bool t_one = t_total <= 512;  // one value per thread
+  float t_val = 0.f;
+  if (t_one && (int)threadIdx.x < t_total) {
+    const int sp = threadIdx.x / a.lora.r, c = threadIdx.x - sp * a.lora.r;
+    t_val = a.lora.t_part[((size_t)sp * M + m) * a.lora.ldt + c];
+  }
+  // the row's own loads (planes, residual)
   float res8[CPT][8];
 #pragma unroll
   for (int i = 0; i < CPT; ++i) {
@@ -215,33 +244,26 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
         for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e]);
         if (a.residual) unpack8(*reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0), res8[i]);
       } else {
+        // the residual is requested before the planes are waited for
+        uint4 r4 = {0, 0, 0, 0};
+        if (a.residual) r4 = *reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0);
         load_base8(a.y_bf16, a.y_part, a.nsplit, m, M, a.D, n0, v[i]);
-        if (a.residual) unpack8(*reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0), res8[i]);
+        if (a.residual) unpack8(r4, res8[i]);
       }
     }
   }
-  // rows of B for this thread's columns and the norm weights: requested now, used after the
-  // barriers below (one row = 16 bytes per thread; up to 16 rows are kept in registers when
-  // every thread owns a single chunk)
-  constexpr int kBR = CPT == 1 ? 16 : 1;
-  const bool lora = !src && a.lora.t_part;
-  const bool b_early = CPT == 1 && lora && a.lora.r <= kBR && (int)threadIdx.x < nchunks;
-  uint4 brow[kBR];
-  if (b_early) {
-#pragma unroll
-    for (int rr = 0; rr < kBR; ++rr)
-      brow[rr] = *reinterpret_cast<const uint4*>(a.lora.b + (size_t)(rr < a.lora.r ? rr : 0) * a.D + threadIdx.x * 8);
-  }
-  uint4 nw4[CPT];
-  if (a.norm_w) {
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = threadIdx.x + 512 * i;
-      nw4[i] = *reinterpret_cast<const uint4*>(a.norm_w + (c < nchunks ? c : 0) * 8);
-    }
-  }
   if (lora) {
-    if (a.lora.r * a.lora.nsplit <= TMX_MAX_LORA_SPLITS * 64) {
+    if (t_one) {
+      // t_s[c] = bf16(sum of the planes' values of column c), planes in ascending order
+      if ((int)threadIdx.x < t_total) t_stage[threadIdx.x] = t_val;
+      __syncthreads();
+      if ((int)threadIdx.x < a.lora.r) {
+        float t = 0.f;
+        for (int sp = 0; sp < a.lora.nsplit; ++sp) t += t_stage[sp * a.lora.r + threadIdx.x];
+        t_s[threadIdx.x] = rbf(t);
+      }
+      __syncthreads();
+    } else if (a.lora.r * a.lora.nsplit <= TMX_MAX_LORA_SPLITS * 64) {
       stage_t_block(t_s, t_stage, a.lora, m, M, 0, a.lora.r);
     } else {
       stage_t(t_s, a.lora, m, M, 0, a.lora.r);
