@@ -11,32 +11,41 @@
 
 namespace tmx {
 
-__global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
-  extern __shared__ float sm[];  // x row [D] | probabilities [E] | partial scores [16][E]
-  __shared__ float red_v[4];
-  __shared__ int red_i[4];
-  __shared__ float sel_w[64];
+constexpr int kRouterThreads = 512, kRowGroups = kRouterThreads / 16;
+
+__global__ __launch_bounds__(kRouterThreads) void moe_router_kernel(RouterArgs a) {
+  extern __shared__ float sm[];  // x row [D] | probabilities [E] | partial scores [kRowGroups][E]
   float* xrow = sm;
   float* prob = sm + a.D;
   const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int d = tid; d < a.D; d += 256) xrow[d] = bf2f(a.x[(size_t)b * a.D + d]);
+  for (int d = tid; d < a.D; d += kRouterThreads) xrow[d] = bf2f(a.x[(size_t)b * a.D + d]);
   __syncthreads();
   // scores: 16 threads cover 128 expert columns of one router row with 16-byte loads (8 experts
-  // each), 16 rows per pass; partial sums over the 16 row groups meet in LDS
-  float* part = prob + a.E;  // [16][E]
+  // each), kRowGroups rows per pass; partial sums over the row groups meet in LDS
+  float* part = prob + a.E;  // [kRowGroups][E]
   for (int e0 = 0; e0 < a.E; e0 += 128) {
     const int eg = (tid & 15) * 8 + e0, dsub = tid >> 4;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (eg < a.E) {
-#pragma unroll 4
-      for (int d = dsub; d < a.D; d += 16) {
-        const uint4 w8 = *reinterpret_cast<const uint4*>(a.w + (size_t)d * a.E + eg);
-        const float xv = xrow[d];
-        const uint32_t ww[4] = {w8.x, w8.y, w8.z, w8.w};
+      // 16 router rows in flight per thread (the loop is bound by the latency of these loads);
+      // rows past D are clamped and weighted by zero
+      for (int d0 = dsub; d0 < a.D; d0 += 16 * kRowGroups) {
+        uint4 w8[16];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          acc[2 * j] = fmaf(xv, bf_lo(ww[j]), acc[2 * j]);
-          acc[2 * j + 1] = fmaf(xv, bf_hi(ww[j]), acc[2 * j + 1]);
+        for (int u = 0; u < 16; ++u) {
+          const int d = d0 + kRowGroups * u;
+          w8[u] = *reinterpret_cast<const uint4*>(a.w + (size_t)(d < a.D ? d : a.D - 1) * a.E + eg);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int d = d0 + kRowGroups * u;
+          const float xv = d < a.D ? xrow[d] : 0.f;
+          const uint32_t ww[4] = {w8[u].x, w8[u].y, w8[u].z, w8[u].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            acc[2 * j] = fmaf(xv, bf_lo(ww[j]), acc[2 * j]);
+            acc[2 * j + 1] = fmaf(xv, bf_hi(ww[j]), acc[2 * j + 1]);
+          }
         }
       }
 #pragma unroll
@@ -44,36 +53,33 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
     }
   }
   __syncthreads();
-  for (int e = tid; e < a.E; e += 256) {
+  for (int e = tid; e < a.E; e += kRouterThreads) {
     float s = 0.f;
 #pragma unroll
-    for (int g = 0; g < 16; ++g) s += part[g * a.E + e];
+    for (int g = 0; g < kRowGroups; ++g) s += part[g * a.E + e];
     prob[e] = rbf(s);
   }
   __syncthreads();
+  // softmax and top-k by the first wave alone (E / 64 values per lane): no barriers between
+  // the k rounds.  Sums run over the experts in the same fixed order on every call.
+  if (wave != 0) return;
   float mx = -INFINITY;
-  for (int e = tid; e < a.E; e += 256) mx = fmaxf(mx, prob[e]);
+  for (int e = lane; e < a.E; e += 64) mx = fmaxf(mx, prob[e]);
   mx = wave_max(mx);
-  if (lane == 0) red_v[wave] = mx;
-  __syncthreads();
-  mx = fmaxf(fmaxf(red_v[0], red_v[1]), fmaxf(red_v[2], red_v[3]));
-  __syncthreads();
   float se = 0.f;
-  for (int e = tid; e < a.E; e += 256) {
+  for (int e = lane; e < a.E; e += 64) {
     const float ex = expf(prob[e] - mx);
     prob[e] = ex;
     se += ex;
   }
-  se = block_sum<4>(se, red_v);
-  __syncthreads();
-  for (int e = tid; e < a.E; e += 256) prob[e] = prob[e] / se;
-  __syncthreads();
+  se = wave_sum(se);
+  for (int e = lane; e < a.E; e += 64) prob[e] = prob[e] / se;
   // top-k by repeated arg-max; among equal probabilities the lower expert id wins
-  float wsum = 0.f;
+  float wsum = 0.f, my_w = 0.f;
   for (int j = 0; j < a.top_k; ++j) {
     float bv = -1.f;
     int bi = 0x7FFFFFFF;
-    for (int e = tid; e < a.E; e += 256) {
+    for (int e = lane; e < a.E; e += 64) {
       const float v = prob[e];
       if (v > bv || (v == bv && e < bi)) { bv = v; bi = e; }
     }
@@ -83,31 +89,20 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
       const int oi = __shfl_xor(bi, off, 64);
       if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
-    if (lane == 0) { red_v[wave] = bv; red_i[wave] = bi; }
-    __syncthreads();
-    bv = red_v[0]; bi = red_i[0];
-#pragma unroll
-    for (int w = 1; w < 4; ++w)
-      if (red_v[w] > bv || (red_v[w] == bv && red_i[w] < bi)) { bv = red_v[w]; bi = red_i[w]; }
-    __syncthreads();
-    if (tid == 0) {
-      a.expert_of[(size_t)b * a.top_k + j] = bi;
-      sel_w[j] = bv;
-      prob[bi] = -2.f;  // taken
-    }
+    if (lane == (bi & 63)) prob[bi] = -2.f;  // taken (the owner lane updates its own element)
+    if (lane == j) { a.expert_of[(size_t)b * a.top_k + j] = bi; my_w = bv; }
     wsum += bv;
-    __syncthreads();
   }
-  if (tid < a.top_k) a.weight_of[(size_t)b * a.top_k + tid] = rbf(sel_w[tid] / wsum);
+  if (lane < a.top_k) a.weight_of[(size_t)b * a.top_k + lane] = rbf(my_w / wsum);
 }
 
 int moe_route(hipStream_t st, const RouterArgs& a, int B) {
   if (!a.x || !a.w || !a.expert_of || !a.weight_of) return TMX_ERR_ARG;
   if (B <= 0 || a.D <= 0 || a.E <= 0 || a.E % 8 || a.top_k <= 0 || a.top_k > 64 || a.top_k > a.E)
     return TMX_ERR_SHAPE;
-  const size_t lds = (size_t)(a.D + 17 * a.E) * sizeof(float);
+  const size_t lds = (size_t)(a.D + (1 + kRowGroups) * a.E) * sizeof(float);
   if (lds > 60000) return TMX_ERR_SHAPE;
-  hipLaunchKernelGGL(moe_router_kernel, dim3(B), dim3(256), lds, st, a);
+  hipLaunchKernelGGL(moe_router_kernel, dim3(B), dim3(kRouterThreads), lds, st, a);
   return check_launch();
 }
 
