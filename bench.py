@@ -270,13 +270,10 @@ def main():
       alg['gate_up_linear'] -= batch * cfg.hidden_dim * 2  # fused SwiGLU: [M, F] goes out, not [M, 2 F]
     # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
     mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
-    # up to 64 rows: K % 256 == 0 below 8192 with fewer than 16 column blocks (or 192 and more)
-    # runs the 4-wave kernel, the rest the direct-to-LDS k-way kernel (K % 256 == 0) or the plain
-    # k-way kernel; above 64 rows the mid-width range starts at 40 column blocks and there is no
-    # direct-to-LDS variant.  An unsplit gate|up runs the fused LoRA + SwiGLU kernel (8 waves up to
-    # 64 rows with K % 512 == 0).
-    mid = 16 if batch <= 64 else 40
-    four = lambda pl: pl.k % 256 == 0 and pl.k < 8192 and not (mid <= (pl.n + 127) // 128 < 192)
+    # K % 256 == 0 below 8192 with fewer than 16 column blocks runs the 4-wave kernel, the rest the
+    # direct-to-LDS k-way kernel (K % 256 == 0) or the plain k-way kernel.  An unsplit gate|up with
+    # LoRA rank <= 16 runs the fused LoRA + SwiGLU kernel (8 waves up to 64 rows with K % 512 == 0).
+    four = lambda pl: pl.k % 256 == 0 and pl.k < 8192 and (pl.n + 127) // 128 < 16
     dense = [('qkv_linear', 'qkv'), ('o_linear', 'o')]
     symbols = {}
     if cfg.num_experts:
@@ -296,7 +293,7 @@ def main():
         dense.append(('gate_up_linear', 'gate_up'))
       dense.append(('down_linear', 'down'))
     def kway_symbol(pl):
-      if batch <= 64 and pl.k % 256 == 0:
+      if pl.k % 256 == 0:
         return f'tmx::qlinear_mfma_dma_kernel<{mt}>'
       return f'tmx::qlinear_mfma_kernel<{mt}, 2>'
     for cls_name, key in dense:

@@ -1080,7 +1080,7 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
 }
 
 template <int MT>
-__global__ __launch_bounds__(512, 2) void qlinear_mfma_dma_kernel(QLinearArgs a) {
+__global__ __launch_bounds__(512, MT == 4 ? 1 : 2) void qlinear_mfma_dma_kernel(QLinearArgs a) {
   extern __shared__ __align__(16) uint16_t smem[];
   if ((int)blockIdx.x >= a.n_main_blocks) gemm_block_dma<MT, true>(a, smem);
   else gemm_block_dma<MT, false>(a, smem);
@@ -1098,17 +1098,12 @@ static int launch_qlinear_dma(hipStream_t st, QLinearArgs a) {
   return check_launch();
 }
 
-// Which kernel serves a projection: the 4-wave kernel needs K % 256 == 0; deep projections
-// (K >= 8192) and mid-width ones (enough column blocks to give every CU a workgroup of 8 waves
-// after the K split, fewer than the 192 from which a projection runs unsplit) go to the k-way
-// kernels.  Up to 64 rows the k-way kernel is the direct-to-LDS one, which wins from 16 column
-// blocks on (measured on the o shapes of the 8B and the 30B-A3B models and on q|k|v); above, from 40.
+// Which kernel serves a projection: narrow ones (fewer than 16 column blocks) with K % 256 == 0
+// below 8192 run the 4-wave kernel; everything else a k-way kernel: the direct-to-LDS one when
+// K % 256 == 0 (measured faster than the 4-wave kernel on the o, q|k|v, down and unsplit gate|up
+// shapes of the 8B and 30B-A3B models at 1, 32, 64 and 128 rows), the plain one otherwise.
 static bool four_wave_shape(int K) { return K % 256 == 0 && K < 8192; }
-static bool four_wave(int K, int N, int M) {
-  const int nblocks = (N + 127) / 128;
-  const int mid = M <= 64 ? 16 : 40;
-  return four_wave_shape(K) && !(nblocks >= mid && nblocks < 192);
-}
+static bool four_wave(int K, int N) { return four_wave_shape(K) && (N + 127) / 128 < 16; }
 
 static int slice_len(int KT, int s) { return ((KT + s - 1) / s + 3) / 4 * 4; }
 static bool slices_ok(int KT, int s) { return (KT + slice_len(KT, s) - 1) / slice_len(KT, s) == s; }
@@ -1134,7 +1129,7 @@ static int num_splits4(int K, int N) {
 
 int qlinear_num_lora_splits(int K, int N);
 int qlinear_num_splits(int K, int N, int M) {
-  if (four_wave(K, N, M)) return num_splits4(K, N);
+  if (four_wave(K, N)) return num_splits4(K, N);
   const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
   // steps of 4 k-tiles (direct-to-LDS kernel up to 64 rows, 128-row kernel) or 8; the workgroups
@@ -1158,9 +1153,7 @@ int qlinear_num_splits(int K, int N, int M) {
 // Number of K-slices of the LoRA projection t = x . A: as fine as whole steps (4 or 8 k-tiles,
 // by kernel) allow, at most TMX_MAX_LORA_SPLITS planes, so that no LoRA block outlasts the
 // main blocks.
-// (the plane count is part of the interface and does not depend on the row count: 8 wherever
-// some row count picks a k-way kernel; the 4-wave kernel takes any multiple of 4)
-static int lora_step(int K, int N) { return four_wave(K, N, 1) ? 4 : 8; }
+static int lora_step(int K, int N) { return four_wave(K, N) ? 4 : 8; }
 int qlinear_num_lora_splits(int K, int N) {
   const int KT = K / 64, g = lora_step(K, N);
   for (int per = g;; per += g) {
@@ -1253,15 +1246,15 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   const int nls = qlinear_num_lora_splits(K, N);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
   a.kt_per_lora_split = lora_slice_len(K, N);
-  if (four_wave(K, N, M)) {
+  if (four_wave(K, N)) {
     if (M <= 32) return launch_qlinear4<1>(st, a);
     if (M <= 64) return launch_qlinear4<2>(st, a);
     return launch_qlinear4<4>(st, a);
   }
   // slices of whole steps, up to 64 rows, 32-bit byte offsets: the direct-to-LDS variant
-  if (M <= 64 && K % 256 == 0 && a.kt_per_split % 4 == 0 && (!a_t || a.kt_per_lora_split % 4 == 0) &&
+  if (K % 256 == 0 && a.kt_per_split % 4 == 0 && (!a_t || a.kt_per_lora_split % 4 == 0) &&
       (size_t)M * ldx * 2 < (1u << 31) && (size_t)K * N / 2 < (1u << 31) && (size_t)K * Rpad * 2 < (1u << 31))
-    return M <= 32 ? launch_qlinear_dma<1>(st, a) : launch_qlinear_dma<2>(st, a);
+    return M <= 32 ? launch_qlinear_dma<1>(st, a) : (M <= 64 ? launch_qlinear_dma<2>(st, a) : launch_qlinear_dma<4>(st, a));
   if (M <= 32) return launch_qlinear<1, 2>(st, a);
   if (M <= 64) return launch_qlinear<2, 2>(st, a);
   return launch_qlinear<4, 2>(st, a);
