@@ -835,9 +835,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
       const int r = kh ? r8 : r8 + 8;
       hb[(((cw * MT + m) * 16 + r) << 6) + lane] = kh ? acc[m][r8] : acc[m][r8 + 8];
     }
-  TMX_STAMP(20);
   __syncthreads();
-  TMX_STAMP(21);
   if constexpr (FUSE) {
     // t = x . [A_gate | A_up]: partial tiles summed in wave order, rounded to bf16, row-major
 #pragma unroll
@@ -850,10 +848,8 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
         for (int w = 0; w < 8; ++w) t += fl[(((w * MT + m) * 16 + r) << 6) + lane];
         ts[(m * 32 + acc_row(r, lane)) * 40 + nl] = f2bf(t);
       }
-    TMX_STAMP(22);
-    __syncthreads();
-    TMX_STAMP(23);
-  }
+      __syncthreads();
+    }
   {
     // y = bf16(x . W) (+ bf16(bf16(t . B) * ls)): the LoRA product runs on the MFMA, t rows as A
     // fragments, the B columns of this tile as B fragments, k = rank padded with zeros
@@ -880,9 +876,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
       }
     }
   }
-  TMX_STAMP(24);
   __syncthreads();
-  TMX_STAMP(25);
   // act = bf16(bf16(g * bf16(sigmoid(g))) * u): every wave finishes a quarter of one gate tile
   {
     const int gt = wave & 1, q = wave >> 1;
