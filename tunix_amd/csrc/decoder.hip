@@ -186,7 +186,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     }
     for (int i = 0; i < m->num_layers; ++i) {
       const tmx_layer_desc& l = m->layers[i];
-      // gate | up with LoRA + SwiGLU in its epilogue: 4-wave kernel shape, unsplit, 2 r <= 32
+      // gate | up with LoRA + SwiGLU in its epilogue: K % 256 == 0 below 8192, unsplit, 2 r <= 32
       const bool fused_gu = !moe && sp.gate_up == 1 && D % 256 == 0 && D < 8192 && F % 64 == 0 &&
                             (!l.gate_up.lora_a_t || (2 * l.gate_up.rank <= 32 && l.gate_up.r_pad == 32));
       uint16_t* kc = (uint16_t*)s->kv_cache + (size_t)(2 * i) * kv_elems;

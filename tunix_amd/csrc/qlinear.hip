@@ -16,9 +16,11 @@
 
 namespace tmx {
 
-// Two kernels share the tile math.  The 4-wave kernel (one wave per column tile, steps of 4
-// k-tiles) serves K % 256 == 0 below 8192; the k-way kernel further down runs two waves per
-// column tile over steps of 8 k-tiles, takes any K % 64 == 0 and serves the deep projections.
+// Three generations of projection kernels share the tile math (the host picks, see four_wave()):
+// the 4-wave block below (narrow projections, the old fused gate|up kernel, the routed experts),
+// the k-way block gemm_block<MT, 2> (any K % 64 == 0), and the direct-to-LDS blocks further down
+// (qlinear_gate_up8_kernel, gemm_block_dma), which carry the decode step wherever K % 256 == 0.
+// The 4-wave block:
 // One workgroup = 4 waves owns a block of 4 adjacent 32-column tiles (one per wave) over one
 // K-slice and advances in steps of KS = 4 k-tiles (256 k).  Per step the activation slab
 // x[0:M, 256 s : 256 s + 256] is fetched once per workgroup with coalesced 16-byte loads
@@ -1126,7 +1128,7 @@ int qlinear_num_splits(int K, int N, int M) {
   if (four_wave(K, N)) return num_splits4(K, N);
   const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
-  // steps of 4 k-tiles (direct-to-LDS kernel up to 64 rows, 128-row kernel) or 8; the workgroups
+  // steps of 4 k-tiles (direct-to-LDS kernel, 128-row k-way kernel) or 8; the workgroups
   // of the LoRA projection share the launch, and a launch that does not fit one workgroup per CU
   // pays a second round (measured: 272 workgroups run slower than 144 with twice the steps); the
   // charge per plane covers the consumer's reads (measured on the o projection: 4 slices beat 6)
