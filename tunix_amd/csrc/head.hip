@@ -159,8 +159,10 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
         } else if (a.mode == TMX_SAMPLE_TOP_P) {
           z = logit / a.temperature;
           if (a.sort_keys) {
-            // ascending key order = descending z (with -0 == +0), rows kept apart by the high word
-            const uint32_t zb = __float_as_uint(z + 0.0f);
+            // ascending key order = descending logit = descending z (T > 0; -0 == +0), rows kept
+            // apart by the high word.  The logit is a bf16 value, so the low 16 key bits only
+            // repeat the sign and the sort leaves them out.
+            const uint32_t zb = __float_as_uint(logit + 0.0f);
             const uint32_t ord = (zb & 0x80000000u) ? ~zb : (zb | 0x80000000u);
             a.sort_keys[(size_t)row * a.V + v] = ((uint64_t)row << 32) | (uint32_t)~ord;
             key = z;

@@ -26,9 +26,11 @@ namespace tmx {
 constexpr int kSelThreads = 1024;
 constexpr int kSelItems = 4;
 
-__device__ __forceinline__ float z_of_key(uint64_t key) {
+// The key's low word orders the bf16 logit (its low 16 bits only repeat the sign, so the sort
+// skips them); z = logit / T is the same f32 division the head kernel makes.
+__device__ __forceinline__ float z_of_key(uint64_t key, float temperature) {
   const uint32_t o = ~(uint32_t)key;
-  return __uint_as_float((o & 0x80000000u) ? (o ^ 0x80000000u) : ~o);
+  return __uint_as_float((o & 0x80000000u) ? (o ^ 0x80000000u) : ~o) / temperature;
 }
 
 __global__ __launch_bounds__(kSelThreads) void nucleus_select_kernel(NucleusArgs a) {
@@ -38,7 +40,7 @@ __global__ __launch_bounds__(kSelThreads) void nucleus_select_kernel(NucleusArgs
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const size_t base = (size_t)row * a.V;
   const int k = a.k;
-  const float z0 = z_of_key(a.keys[base]);
+  const float z0 = z_of_key(a.keys[base], a.temperature);
 
   // full-vocabulary log-sum-exp from the head kernel's per-workgroup partials
   float mx = kNegBig, se = 0.f;
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(kSelThreads) void nucleus_select_kernel(NucleusArgs
   }
   // softmax denominator over the k candidates
   float s = 0.f;
-  for (int i = tid; i < k; i += kSelThreads) s += expf(z_of_key(a.keys[base + i]) - z0);
+  for (int i = tid; i < k; i += kSelThreads) s += expf(z_of_key(a.keys[base + i], a.temperature) - z0);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     lse_merge(mx, se, __shfl_xor(mx, off, 64), __shfl_xor(se, off, 64));
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(kSelThreads) void nucleus_select_kernel(NucleusArgs
 #pragma unroll
     for (int j = 0; j < kSelItems; ++j) {
       const int i = i0 + j;
-      z[j] = i < k ? z_of_key(a.keys[base + i]) : -INFINITY;
+      z[j] = i < k ? z_of_key(a.keys[base + i], a.temperature) : -INFINITY;
       p[j] = i < k ? expf(z[j] - z0) / denom : 0.f;
       t += p[j];
     }
@@ -146,7 +148,7 @@ static int row_bits(int M) {
 static hipError_t sort_rows(void* tmp, size_t& tmp_bytes, const uint64_t* kin, uint64_t* kout,
                             uint32_t* vout, int M, int V, hipStream_t st) {
   return rocprim::radix_sort_pairs(tmp, tmp_bytes, kin, kout, rocprim::counting_iterator<uint32_t>(0),
-                                   vout, (size_t)M * V, 0u, (unsigned)(32 + row_bits(M)), st, false);
+                                   vout, (size_t)M * V, 16u, (unsigned)(32 + row_bits(M)), st, false);
 }
 
 // keys in | keys out | values out | sort scratch
@@ -196,6 +198,7 @@ int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void
   n.M = a.M; n.V = a.V;
   n.k = (top_k > 0 && top_k < a.V) ? top_k : a.V;
   n.top_p = top_p;
+  n.temperature = a.temperature;
   n.k0 = a.k0; n.k1 = a.k1;
   n.step = a.step;
   n.part_f = a.part_f; n.nwg = a.nwg;

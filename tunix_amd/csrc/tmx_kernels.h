@@ -161,6 +161,7 @@ struct NucleusArgs {
   const uint32_t* vals;  // [M, V] linear index row * V + v of each sorted key
   int M, V, k;           // k: candidates kept by top-k (V without top-k)
   float top_p;
+  float temperature;     // the keys order the bf16 logits; z = logit / temperature
   uint32_t k0, k1;
   const int32_t* step;
   const float* part_f;   // head partials [M][nwg][4]
