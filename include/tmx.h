@@ -45,6 +45,7 @@ extern "C" {
 #define TMX_MAX_RPAD 128   /* widest padded LoRA projection (sum of fused ranks, rounded up to 32) */
 #define TMX_MAX_SPLITS 16  /* most K-slices a projection is split into */
 #define TMX_MAX_LORA_SPLITS 32 /* most K-slices of the LoRA projection x . A */
+#define TMX_MAX_FILL_ROWS 4096 /* most rows (sequences x tokens) of one cache-fill pass */
 
 #define TMX_SAMPLE_GREEDY 0
 #define TMX_SAMPLE_TOP_P 1
@@ -61,7 +62,8 @@ int tmx_abi_version(void);
 int tmx_int4_dequant(void* stream, const void* qweight, const void* scales, void* w_out, int K, int N,
                      int G);
 
-/* y[M, N] = bf16(x[M, K] . dequant(qweight)) (+ LoRA delta) (+ residual), M <= 128.
+/* y[M, N] = bf16(x[M, K] . dequant(qweight)) (+ LoRA delta) (+ residual).  Up to 128 rows run
+ * the decode kernels (K % 64 == 0); more rows run in 256-row blocks and need K % 128 == 0.
  * Replaces the qwix-wrapped Einsum / nnx.Linear call: tunix/models/llama3/model.py:216-218,
  * :489-496; tunix/models/qwen3/model.py:389-393, :1199-1208.
  *   lora_a_t : A in MFMA fragment order, bf16 [K/64][r_pad/32][4][64][8], r_pad % 32 == 0,
@@ -258,8 +260,11 @@ typedef struct {
   size_t nucleus_workspace_bytes;
   int tokens_per_pass;     /* 0 or 1: one token per sequence and step.  T > 1 (cache fill with
                               sample == 0, or TMX_SAMPLE_SCORE): every pass consumes the T tokens at
-                              columns *step .. *step + T - 1 of each sequence as batch * T rows (<= 128),
-                              each attending to the slots up to its own column; *step advances by T.
+                              columns *step .. *step + T - 1 of each sequence as batch * T rows, each
+                              attending to the slots up to its own column; *step advances by T.
+                              Rows: <= 128 when scoring or for MoE models; a cache fill of a dense
+                              model takes up to TMX_MAX_FILL_ROWS when every projection has
+                              K % 128 == 0.
                               The workspace must be sized for batch * T rows. */
 } tmx_decode_state;
 

@@ -50,7 +50,7 @@ def test_argument_checks_return_codes_without_a_gpu():
   assert lib.tmx_int4_dequant(None, 1, 1, 1, 65, 32, 64) == -2
   assert lib.tmx_qlora_linear(None, None, None, None, None, None, None, None, None, 1, 64, 32, 64, 0, 0, 0.0) == -1
   assert lib.tmx_qlora_linear_planes(None, 1, 1, 1, None, 1, None, 4, 100, 32, 64, 0, 1) == -2
-  assert lib.tmx_qlora_linear_planes(None, 1, 1, 1, None, 1, None, 200, 128, 32, 64, 0, 1) == -2
+  assert lib.tmx_qlora_linear_planes(None, 1, 1, 1, None, 1, None, 200, 192, 32, 64, 0, 1) == -2  # more than 128 rows: K % 128
   assert lib.tmx_decode_steps(None, None, None, 1, 1) == -1
   assert lib.tmx_head_sample_workspace_bytes(4, 1024) == 4 * 8 * 5 * 4
   assert lib.tmx_qlora_linear_num_splits(64, 4096, 4096) >= 1

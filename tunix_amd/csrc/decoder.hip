@@ -120,7 +120,9 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   if (NSEQ <= 0 || NSEQ > 128 || T > 128) return TMX_ERR_SHAPE;
   if (T > 1 && sample && s->sampling_mode != TMX_SAMPLE_SCORE) return TMX_ERR_ARG;
   const int B = NSEQ * T, C = s->cache_size, L = s->buf_len;
-  if (B > 128 || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
+  // sampling (the head) takes up to 128 rows; a cache-fill pass of a dense model up to
+  // TMX_MAX_FILL_ROWS, which the projections multiply in 256-row blocks (every K % 128 == 0)
+  if (B > ((sample || moe) ? 128 : TMX_MAX_FILL_ROWS) || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
   if (moe && (m->experts_per_tok <= 0 || m->experts_per_tok > m->num_experts ||
               (size_t)B * m->experts_per_tok > 1024))
     return TMX_ERR_SHAPE;
@@ -187,7 +189,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     for (int i = 0; i < m->num_layers; ++i) {
       const tmx_layer_desc& l = m->layers[i];
       // gate | up with LoRA + SwiGLU in its epilogue: K % 256 == 0 below 8192, unsplit, 2 r <= 32
-      const bool fused_gu = !moe && sp.gate_up == 1 && D % 256 == 0 && D < 8192 && F % 64 == 0 &&
+      const bool fused_gu = !moe && B <= 128 && sp.gate_up == 1 && D % 256 == 0 && D < 8192 && F % 64 == 0 &&
                             (!l.gate_up.lora_a_t || (2 * l.gate_up.rank <= 32 && l.gate_up.r_pad == 32));
       uint16_t* kc = (uint16_t*)s->kv_cache + (size_t)(2 * i) * kv_elems;
       uint16_t* vc = kc + kv_elems;

@@ -1094,6 +1094,171 @@ static int launch_qlinear_dma(hipStream_t st, QLinearArgs a) {
   return check_launch();
 }
 
+// ---------------------------------------------------------------------------
+// Many rows (cache fill over whole prompts: more than 128 rows per pass).  A workgroup owns 256
+// rows x 128 columns, so every dequantised weight fragment feeds 8 MFMAs instead of 1..4 and the
+// loop is bound by the matrix pipe, not by dequantisation: wave (ct, kw) multiplies column tile
+// ct by k-tile kw of every 2-tile step against all 8 row tiles (128 accumulator registers).  Same
+// buffer loads and direct-to-LDS slab as the k-way block above, with 256-byte slab rows (four
+// rows per 1 KiB transfer), chunks XOR-swizzled by row % 16.  Two waves per SIMD: one dequantises
+// while the other multiplies.  Row blocks are blockIdx.z; K-slices (blockIdx.y) work as above.
+struct KW {
+  static constexpr int MT = 8, ROWS = 256, TS = 2, XS = 128;
+  static constexpr size_t LDS = (size_t)2 * ROWS * XS * 2;  // 128 KiB, also holds the reduction
+};
+
+template <bool LORA>
+__device__ __forceinline__ void gemm_block_wide(const QLinearArgs& a, uint16_t* smem) {
+  constexpr int MT = KW::MT, TS = KW::TS, XS = KW::XS, ROWS = KW::ROWS;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), ct = wave & 3, kw = wave >> 2;
+  const int h = lane >> 5, nl = lane & 31;
+  const int KT = a.K >> 6;
+  const int slice = LORA ? ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y
+                         : (int)blockIdx.y;
+  const int per = LORA ? a.kt_per_lora_split : a.kt_per_split;
+  const int kb0 = slice * per;
+  const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
+  const int nsteps = (kb1 - kb0) / TS, last_step = nsteps - 1;  // host: whole steps
+  if (nsteps <= 0) return;
+  const int row0 = (int)blockIdx.z * ROWS;
+  const int rows = a.M - row0 < ROWS ? a.M - row0 : ROWS;  // host: >= 1
+  const int gs = __builtin_ctz(a.G >> 6), KG = a.K / a.G;
+  const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
+  const int nb = LORA ? ct : (int)blockIdx.x * 4 + ct;
+  const bool tile_ok = nb < NT;  // waves past the last tile only help with the slab
+
+  const __amdgpu_buffer_rsrc_t rw =
+      LORA ? make_rsrc(a.a_t, (uint32_t)KT * NT * 4096u) : make_rsrc(a.qw, (uint32_t)NT * KT * 1024u);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scales, LORA ? 0u : (uint32_t)NT * KG * 64u);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x + (size_t)row0 * a.ldx, (uint32_t)rows * a.ldx * 2u);
+  const int wv = LORA ? nb * 4096 + lane * 16 : (nb * KT * 64 + lane) * 16;
+  const int wstep = LORA ? NT * 4096 : 1024;  // bytes between consecutive k-tiles
+  const int sv = (nb * KG * 32 + nl) * 2;
+  // slab transfer: 8 loads per wave and step; load i moves rows 4 wave + 32 i .. + 3 (16 lanes
+  // each), lane l delivering chunk (l % 16) ^ (row % 16) of the step to slot l % 16
+  constexpr int XR = ROWS / 32;
+  int xoff[XR];  // per-lane byte offset in the row block (rows past the end repeat the last)
+#pragma unroll
+  for (int i = 0; i < XR; ++i) {
+    const int row_l = 4 * wave + 32 * i + (lane >> 4);
+    xoff[i] = (row_l < rows ? row_l : rows - 1) * a.ldx * 2 + (((lane & 15) ^ (row_l & 15)) * 16) + kb0 * 128;
+  }
+
+  f32x16_t acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
+  constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
+  u32x4_t wring[WPT];
+  uint16_t sring = 0;
+
+  auto load_w_tile = [&](int step) __attribute__((always_inline)) {
+    step = step < last_step ? step : last_step;
+    const int kt = kb0 + step * TS + kw;
+#pragma unroll
+    for (int t = 0; t < WPT; ++t) wring[t] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv + t * 1024, kt * wstep, 0);
+    if (!LORA) sring = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
+  };
+  auto dma_x = [&](int step, int buf) __attribute__((always_inline)) {
+    step = step < last_step ? step : last_step;
+    uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * 4 * XS;
+#pragma unroll
+    for (int i = 0; i < XR; ++i) load_row_to_lds(rx, base + i * 32 * XS, xoff[i], step * (TS * 128));
+  };
+  auto tile_math = [&](int step, int buf) __attribute__((always_inline)) {
+    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + nl * XS;
+    u32x4_t wc[WPT];
+#pragma unroll
+    for (int t = 0; t < WPT; ++t) wc[t] = wring[t];
+    const float s_c = LORA ? 0.f : bf2f(sring);
+    load_w_tile(step + 1);  // registers consumed: refill them one step ahead
+    const float m8s = -8.f * s_c;
+    const uint32_t wd[4] = {wc[0].x, wc[0].y, wc[0].z, wc[0].w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      // chunk 8 kw + 2 t + h of the row sits at slot (8 kw + 2 t + h) ^ (row % 16)
+      const int slot = ((8 * kw + 2 * t + h) ^ (nl & 15)) * 8;
+      bf16x8_t xa[MT];
+#pragma unroll
+      for (int m = 0; m < MT; ++m) xa[m] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + slot);
+      bf16x8_t b;
+      if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[t % WPT]);
+      else b = dequant_word(wd[t], s_c, m8s);
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m], b, acc[m], 0, 0, 0);
+    }
+  };
+  // loads of a step younger than its slab transfer (in-order counter)
+  constexpr int kYounger = LORA ? 4 : 2;
+  auto wait_slab = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    if (tile_ok) __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  };
+
+  dma_x(0, 0);
+  if (tile_ok) load_w_tile(0);
+  wait_slab();
+  for (int step = 0; step < nsteps; ++step) {
+    const int buf = step & 1;
+    dma_x(step + 1, buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (tile_ok) tile_math(step, buf);
+    wait_slab();
+  }
+
+  // the two k-halves of a tile swap halves of their accumulators through LDS (the slab is free:
+  // the last step ended with a barrier): the first finishes registers 0..7, the second 8..15
+  float* hb = reinterpret_cast<float*>(smem);  // [4 tiles][MT][16][64]: all of the slab's 128 KiB
+  if (tile_ok) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r8 = 0; r8 < 8; ++r8) {
+        const int r = kw ? r8 : r8 + 8;
+        hb[(((ct * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
+      }
+  }
+  __syncthreads();
+  if (!tile_ok) return;
+  const int col = nb * 32 + nl;
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r8 = 0; r8 < 8; ++r8) {
+      const int r = kw ? r8 + 8 : r8;
+      const int row = row0 + m * 32 + acc_row(r, lane);
+      if (row >= a.M) continue;
+      const float mine = acc[m][r], other = hb[(((ct * MT + m) * 16 + r) << 6) + lane];
+      const float v = kw ? other + mine : mine + other;  // first half + second half
+      if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = v;
+      else if (a.y_bf16) a.y_bf16[(size_t)row * a.ldy + col] = f2bf(v);
+      else a.y_part[((size_t)slice * a.M + row) * a.N + col] = v;
+    }
+}
+
+__global__ __launch_bounds__(512, 1) void qlinear_mfma_wide_kernel(QLinearArgs a) {
+  extern __shared__ __align__(16) uint16_t smem[];
+  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block_wide<true>(a, smem);
+  else gemm_block_wide<false>(a, smem);
+}
+
+static int launch_qlinear_wide(hipStream_t st, QLinearArgs a) {
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&qlinear_mfma_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+      (int)KW::LDS);
+  if (attr != hipSuccess) return TMX_ERR_LAUNCH;
+  a.n_main_blocks = (a.N + 127) / 128;
+  const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
+  const int row_blocks = (a.M + KW::ROWS - 1) / KW::ROWS;
+  hipLaunchKernelGGL(qlinear_mfma_wide_kernel, dim3(blocks, a.nsplit, row_blocks), dim3(512), KW::LDS, st, a);
+  return check_launch();
+}
+
 // Which kernel serves a projection: narrow ones (fewer than 16 column blocks) with K % 256 == 0
 // below 8192 run the 4-wave kernel; everything else a k-way kernel: the direct-to-LDS one when
 // K % 256 == 0 (measured faster than the 4-wave kernel on the o, q|k|v, down and unsplit gate|up
@@ -1125,6 +1290,13 @@ static int num_splits4(int K, int N) {
 
 int qlinear_num_lora_splits(int K, int N);
 int qlinear_num_splits(int K, int N, int M) {
+  if (M > 128) {
+    // 256-row blocks: K-slices only while the launch has fewer workgroups than CUs
+    const int wgs = (N + 127) / 128 * ((M + 255) / 256);
+    int s = 1;
+    while (wgs * s < 192 && s * 2 <= TMX_MAX_SPLITS && slices_ok(K / 64, s * 2) && slice_len(K / 64, s * 2) >= 8) s *= 2;
+    return s;
+  }
   if (four_wave(K, N)) return num_splits4(K, N);
   const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
@@ -1218,7 +1390,7 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
                  int N, int G, int Rpad, int nsplit) {
   if (!x || !qw || !scales || (!y_bf16 && !y_part)) return TMX_ERR_ARG;
-  if (M <= 0 || M > 128 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
+  if (M <= 0 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
   if (K % 64 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
   if (a_t && (!t_part || Rpad <= 0 || Rpad % 32 || Rpad > 128 || ldt < Rpad)) return TMX_ERR_SHAPE;
   if (nsplit < 1 || nsplit > TMX_MAX_SPLITS || (nsplit > 1 && !y_part)) return TMX_ERR_ARG;
@@ -1242,6 +1414,13 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   const int nls = qlinear_num_lora_splits(K, N);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
   a.kt_per_lora_split = lora_slice_len(K, N);
+  if (M > 128) {
+    // more than 128 rows: the 256-row block (whole 2-tile steps, 32-bit byte offsets per row block)
+    if (K % 128 || a.kt_per_split % 2 || (a_t && a.kt_per_lora_split % 2) || (size_t)256 * ldx * 2 >= (1u << 31) ||
+        (size_t)K * N / 2 >= (1u << 31) || (size_t)K * Rpad * 2 >= (1u << 31))
+      return TMX_ERR_SHAPE;
+    return launch_qlinear_wide(st, a);
+  }
   if (four_wave(K, N)) {
     if (M <= 32) return launch_qlinear4<1>(st, a);
     if (M <= 64) return launch_qlinear4<2>(st, a);
@@ -1347,7 +1526,7 @@ extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight
   const bool lora = lora_a_t != nullptr;
   if (!workspace || !y) return TMX_ERR_ARG;
   if (lora && (!lora_b || r <= 0 || r > r_pad)) return TMX_ERR_ARG;
-  if (M <= 0 || M > 128) return TMX_ERR_SHAPE;
+  if (M <= 0) return TMX_ERR_SHAPE;
   const int ns = qlinear_num_splits(K, N, M);
   float* y_part = (float*)workspace;
   float* t_part = y_part + (size_t)ns * M * N;

@@ -221,14 +221,22 @@ class Sampler:
       s.nucleus_workspace, s.nucleus_workspace_bytes = self._nucleus_ws.data_ptr(), self._nucleus_ws.numel()
     return s
 
-  MAX_ROWS = 128  # rows of one pass the kernels take (sequences x tokens per pass)
+  MAX_ROWS = 128        # rows of one pass with the head (sequences x tokens per pass)
+  MAX_FILL_ROWS = 2048  # rows of one cache-fill pass of a dense model (256-row projection blocks)
+
+  def _fill_rows(self):
+    cfg = self._transformer.config
+    ks = (cfg.embed_dim, cfg.num_heads * cfg.head_dim, cfg.hidden_dim)
+    wide = not cfg.num_experts and all(k % 128 == 0 for k in ks)
+    return self.MAX_FILL_ROWS if wide else self.MAX_ROWS
 
   def walk(self, st, n_tokens, sample=False):
     """Advances every sequence by n_tokens known tokens (cache fill over a prompt, or scoring
     when st['sampling_mode'] == 'score') in passes of as many tokens per sequence as fit
-    MAX_ROWS rows, instead of one token per launch sequence."""
+    MAX_ROWS rows (MAX_FILL_ROWS without the head, where the model allows), instead of one
+    token per launch sequence."""
     b = st['token_buffer'].shape[0]
-    per = max(1, self.MAX_ROWS // b)
+    per = min(128, max(1, (self.MAX_ROWS if sample else self._fill_rows()) // b))
     while n_tokens > 0:
       t = min(per, n_tokens)
       self.run_steps(st, 1, sample=sample, tokens_per_pass=t)
