@@ -1095,37 +1095,37 @@ static int launch_qlinear_dma(hipStream_t st, QLinearArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Many rows (cache fill over whole prompts: more than 128 rows per pass).  A workgroup owns 256
-// rows x 128 columns, so every dequantised weight fragment feeds 8 MFMAs instead of 1..4 and the
-// loop is bound by the matrix pipe, not by dequantisation: wave (ct, kw) multiplies column tile
-// ct by k-tile kw of every 2-tile step against all 8 row tiles (128 accumulator registers).  Same
-// buffer loads and direct-to-LDS slab as the k-way block above, with 256-byte slab rows (four
-// rows per 1 KiB transfer), chunks XOR-swizzled by row % 16.  Two waves per SIMD: one dequantises
-// while the other multiplies.  Row blocks are blockIdx.z; K-slices (blockIdx.y) work as above.
+// Many rows (cache fill over whole prompts: more than 128 rows per pass).  At this size the
+// bound is what a CU can pull through its vector memory path (about 30 GB/s per CU, L2 hits
+// included), so the block is as large as the registers allow: 256 rows x 256 columns, 0.31 bytes
+// loaded per kFLOP.  Wave ct owns column tile ct and multiplies both k-tiles of every 2-tile step
+// against all 8 row tiles (128 accumulator registers), so a dequantised weight fragment feeds 8
+// MFMAs.  Same buffer loads and direct-to-LDS slab as the k-way block above, with 256-byte slab
+// rows (four rows per 1 KiB transfer), chunks XOR-swizzled by row % 16.  Two waves per SIMD: one
+// dequantises while the other multiplies.  Row blocks are blockIdx.z, K-slices blockIdx.y.
 struct KW {
-  static constexpr int MT = 8, ROWS = 256, TS = 2, XS = 128;
-  static constexpr size_t LDS = (size_t)2 * ROWS * XS * 2;  // 128 KiB, also holds the reduction
+  static constexpr int MT = 8, ROWS = 256, COLS = 256, TS = 2, XS = 128;
+  static constexpr size_t LDS = (size_t)2 * ROWS * XS * 2;  // 128 KiB
 };
 
 template <bool LORA>
-__device__ __forceinline__ void gemm_block_wide(const QLinearArgs& a, uint16_t* smem) {
+__device__ __forceinline__ void gemm_block_wide(const QLinearArgs& a, uint16_t* smem, int bx, int by, int bz) {
   constexpr int MT = KW::MT, TS = KW::TS, XS = KW::XS, ROWS = KW::ROWS;
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), ct = wave & 3, kw = wave >> 2;
+  const int ct = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, nl = lane & 31;
   const int KT = a.K >> 6;
-  const int slice = LORA ? ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y
-                         : (int)blockIdx.y;
+  const int slice = LORA ? (bx - a.n_main_blocks) + a.lora_blocks_per_split * by : by;
   const int per = LORA ? a.kt_per_lora_split : a.kt_per_split;
   const int kb0 = slice * per;
   const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
   const int nsteps = (kb1 - kb0) / TS, last_step = nsteps - 1;  // host: whole steps
   if (nsteps <= 0) return;
-  const int row0 = (int)blockIdx.z * ROWS;
+  const int row0 = bz * ROWS;
   const int rows = a.M - row0 < ROWS ? a.M - row0 : ROWS;  // host: >= 1
   const int gs = __builtin_ctz(a.G >> 6), KG = a.K / a.G;
   const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
-  const int nb = LORA ? ct : (int)blockIdx.x * 4 + ct;
+  const int nb = LORA ? ct : bx * 8 + ct;
   const bool tile_ok = nb < NT;  // waves past the last tile only help with the slab
 
   const __amdgpu_buffer_rsrc_t rw =
@@ -1141,7 +1141,7 @@ __device__ __forceinline__ void gemm_block_wide(const QLinearArgs& a, uint16_t* 
   int xoff[XR];  // per-lane byte offset in the row block (rows past the end repeat the last)
 #pragma unroll
   for (int i = 0; i < XR; ++i) {
-    const int row_l = 4 * wave + 32 * i + (lane >> 4);
+    const int row_l = 4 * ct + 32 * i + (lane >> 4);
     xoff[i] = (row_l < rows ? row_l : rows - 1) * a.ldx * 2 + (((lane & 15) ^ (row_l & 15)) * 16) + kb0 * 128;
   }
 
@@ -1151,48 +1151,82 @@ __device__ __forceinline__ void gemm_block_wide(const QLinearArgs& a, uint16_t* 
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
   constexpr int WPT = LORA ? 4 : 1;  // 16-byte words per lane and tile
-  u32x4_t wring[WPT];
-  uint16_t sring = 0;
+  u32x4_t wring[TS][WPT];
+  uint16_t sring[TS];
 
-  auto load_w_tile = [&](int step) __attribute__((always_inline)) {
+  auto load_w_tile = [&](int step, auto jc) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
     step = step < last_step ? step : last_step;
-    const int kt = kb0 + step * TS + kw;
+    const int kt = kb0 + step * TS + j;
 #pragma unroll
-    for (int t = 0; t < WPT; ++t) wring[t] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv + t * 1024, kt * wstep, 0);
-    if (!LORA) sring = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
+    for (int t = 0; t < WPT; ++t) wring[j][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, wv + t * 1024, kt * wstep, 0);
+    if (!LORA) sring[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, sv, (kt >> gs) * 64, 0);
   };
   auto dma_x = [&](int step, int buf) __attribute__((always_inline)) {
     step = step < last_step ? step : last_step;
-    uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * 4 * XS;
+    uint16_t* base = smem + (size_t)buf * ROWS * XS + ct * 4 * XS;
 #pragma unroll
     for (int i = 0; i < XR; ++i) load_row_to_lds(rx, base + i * 32 * XS, xoff[i], step * (TS * 128));
   };
-  auto tile_math = [&](int step, int buf) __attribute__((always_inline)) {
+  // One step: 8 fragment groups g = 4 j + t (k-tile j, 16-wide k-block t) of 8 MFMAs, one per row
+  // tile.  Between the MFMAs of group g the wave reads the x fragments of group g + 1 (one LDS
+  // read per MFMA; chunk 2 g + h of a row sits at slot (2 g + h) ^ (row % 16)) and dequantises its
+  // weight fragment a quarter at a time, so the matrix pipe waits neither for LDS nor for the
+  // VALU, also when both waves of a SIMD run in phase after a barrier.  The order is pinned.
+  auto step_math = [&](int step, int buf) __attribute__((always_inline)) {
+    u32x4_t wc[TS][WPT];
+    float s_c[TS], m8s[TS];
+    static_for<TS>([&](auto jc) __attribute__((always_inline)) {
+      constexpr int j = decltype(jc)::value;
+#pragma unroll
+      for (int t = 0; t < WPT; ++t) wc[j][t] = wring[j][t];
+      s_c[j] = LORA ? 0.f : bf2f(sring[j]);
+      m8s[j] = -8.f * s_c[j];
+      load_w_tile(step + 1, jc);  // registers consumed: refill them one step ahead
+    });
     const uint16_t* xb = smem + (size_t)buf * ROWS * XS + nl * XS;
-    u32x4_t wc[WPT];
+    auto word_of = [&](auto gc) __attribute__((always_inline)) {
+      constexpr int g = decltype(gc)::value, j = g / 4, t = g % 4;
+      return t == 0 ? wc[j][0].x : (t == 1 ? wc[j][0].y : (t == 2 ? wc[j][0].z : wc[j][0].w));
+    };
+    bf16x8_t xq[2][MT];
+    u32x4_t bq[2];
+    {
+      const int slot = (h ^ (nl & 15)) * 8;
 #pragma unroll
-    for (int t = 0; t < WPT; ++t) wc[t] = wring[t];
-    const float s_c = LORA ? 0.f : bf2f(sring);
-    load_w_tile(step + 1);  // registers consumed: refill them one step ahead
-    const float m8s = -8.f * s_c;
-    const uint32_t wd[4] = {wc[0].x, wc[0].y, wc[0].z, wc[0].w};
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      // chunk 8 kw + 2 t + h of the row sits at slot (8 kw + 2 t + h) ^ (row % 16)
-      const int slot = ((8 * kw + 2 * t + h) ^ (nl & 15)) * 8;
-      bf16x8_t xa[MT];
-#pragma unroll
-      for (int m = 0; m < MT; ++m) xa[m] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + slot);
-      bf16x8_t b;
-      if (LORA) b = __builtin_bit_cast(bf16x8_t, wc[t % WPT]);
-      else b = dequant_word(wd[t], s_c, m8s);
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m], b, acc[m], 0, 0, 0);
+      for (int m = 0; m < MT; ++m) xq[0][m] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + slot);
+      if (LORA) bq[0] = wc[0][0];
+      else bq[0] = __builtin_bit_cast(u32x4_t, dequant_word(word_of(IC<0>{}), s_c[0], m8s[0]));
     }
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<4 * TS>([&](auto gc) __attribute__((always_inline)) {
+      constexpr int g = decltype(gc)::value, cur = g & 1, nxt = cur ^ 1;
+      constexpr bool more = g + 1 < 4 * TS;
+      constexpr int jn = (g + 1) / 4 % TS, tn = (g + 1) % 4;
+      const int slot = ((2 * (g + 1) + h) ^ (nl & 15)) * 8;
+      uint32_t lo = 0, hi = 0;
+      static_for<MT>([&](auto mc) __attribute__((always_inline)) {
+        constexpr int m = decltype(mc)::value;
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xq[cur][m], __builtin_bit_cast(bf16x8_t, bq[cur]), acc[m],
+                                                         0, 0, 0);
+        if constexpr (more) {
+          xq[nxt][m] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + slot);
+          if (LORA) {
+            if (m == 0) bq[nxt] = wc[jn][tn % WPT];
+          } else {
+            if (m == 0) dequant_masks(word_of(IC<g + 1>{}), lo, hi);
+            if (m == 1) bq[nxt].x = dequant_part<0>(lo, hi, s_c[jn], m8s[jn]);
+            if (m == 2) bq[nxt].y = dequant_part<1>(lo, hi, s_c[jn], m8s[jn]);
+            if (m == 3) bq[nxt].z = dequant_part<2>(lo, hi, s_c[jn], m8s[jn]);
+            if (m == 4) bq[nxt].w = dequant_part<3>(lo, hi, s_c[jn], m8s[jn]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+    });
   };
   // loads of a step younger than its slab transfer (in-order counter)
-  constexpr int kYounger = LORA ? 4 : 2;
+  constexpr int kYounger = TS * (LORA ? 4 : 2);
   auto wait_slab = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_sched_barrier(0);
     if (tile_ok) __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
@@ -1201,50 +1235,45 @@ __device__ __forceinline__ void gemm_block_wide(const QLinearArgs& a, uint16_t* 
   };
 
   dma_x(0, 0);
-  if (tile_ok) load_w_tile(0);
+  if (tile_ok) static_for<TS>([&](auto jc) __attribute__((always_inline)) { load_w_tile(0, jc); });
   wait_slab();
   for (int step = 0; step < nsteps; ++step) {
     const int buf = step & 1;
     dma_x(step + 1, buf ^ 1);
     __builtin_amdgcn_sched_barrier(0);
-    if (tile_ok) tile_math(step, buf);
+    if (tile_ok) step_math(step, buf);
     wait_slab();
   }
-
-  // the two k-halves of a tile swap halves of their accumulators through LDS (the slab is free:
-  // the last step ended with a barrier): the first finishes registers 0..7, the second 8..15
-  float* hb = reinterpret_cast<float*>(smem);  // [4 tiles][MT][16][64]: all of the slab's 128 KiB
-  if (tile_ok) {
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int r8 = 0; r8 < 8; ++r8) {
-        const int r = kw ? r8 : r8 + 8;
-        hb[(((ct * MT + m) * 16 + r) << 6) + lane] = acc[m][r];
-      }
-  }
-  __syncthreads();
   if (!tile_ok) return;
   const int col = nb * 32 + nl;
 #pragma unroll
   for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int r8 = 0; r8 < 8; ++r8) {
-      const int r = kw ? r8 + 8 : r8;
+    for (int r = 0; r < 16; ++r) {
       const int row = row0 + m * 32 + acc_row(r, lane);
       if (row >= a.M) continue;
-      const float mine = acc[m][r], other = hb[(((ct * MT + m) * 16 + r) << 6) + lane];
-      const float v = kw ? other + mine : mine + other;  // first half + second half
+      const float v = acc[m][r];
       if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = v;
       else if (a.y_bf16) a.y_bf16[(size_t)row * a.ldy + col] = f2bf(v);
       else a.y_part[((size_t)slice * a.M + row) * a.N + col] = v;
     }
 }
 
-__global__ __launch_bounds__(512, 1) void qlinear_mfma_wide_kernel(QLinearArgs a) {
+// Workgroups are dispatched round-robin over the 8 XCDs (linear id % 8), each with its own L2.
+// The launch is one-dimensional and maps ids so that the workgroups of an XCD share row blocks:
+// with S = gcd(row blocks, 8), XCD x works on row blocks x % S, x % S + S, ... in turn, all column
+// blocks and K-slices of one before the next, so the activation slab of a step is fetched into
+// that L2 once and the other workgroups of the XCD hit it.  Ids past the end do nothing.
+__global__ __launch_bounds__(512, 1) void qlinear_mfma_wide_kernel(QLinearArgs a, int blocks, int row_blocks, int S) {
   extern __shared__ __align__(16) uint16_t smem[];
-  if ((int)blockIdx.x >= a.n_main_blocks) gemm_block_wide<true>(a, smem);
-  else gemm_block_wide<false>(a, smem);
+  const int id = (int)blockIdx.x, xcd = id & 7, idx = id >> 3;
+  const int per_rb = blocks * a.nsplit;
+  const int p = xcd / S + (8 / S) * idx;
+  const int bz = xcd % S + S * (p / per_rb);
+  if (bz >= row_blocks) return;
+  const int cb = p % per_rb, bx = cb % blocks, by = cb / blocks;
+  if (bx >= a.n_main_blocks) gemm_block_wide<true>(a, smem, bx, by, bz);
+  else gemm_block_wide<false>(a, smem, bx, by, bz);
 }
 
 static int launch_qlinear_wide(hipStream_t st, QLinearArgs a) {
@@ -1252,10 +1281,15 @@ static int launch_qlinear_wide(hipStream_t st, QLinearArgs a) {
       reinterpret_cast<const void*>(&qlinear_mfma_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
       (int)KW::LDS);
   if (attr != hipSuccess) return TMX_ERR_LAUNCH;
-  a.n_main_blocks = (a.N + 127) / 128;
+  a.n_main_blocks = (a.N + KW::COLS - 1) / KW::COLS;
   const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
   const int row_blocks = (a.M + KW::ROWS - 1) / KW::ROWS;
-  hipLaunchKernelGGL(qlinear_mfma_wide_kernel, dim3(blocks, a.nsplit, row_blocks), dim3(512), KW::LDS, st, a);
+  int S = 8;
+  while (row_blocks % S) S >>= 1;  // gcd(row_blocks, 8)
+  // ids cover 8 / S XCDs x (row_blocks / S) row blocks x blocks x nsplit per residue, rounded up to 8
+  const long total = (long)blocks * a.nsplit * row_blocks;
+  const int ids = (int)((total + 7) / 8 * 8);
+  hipLaunchKernelGGL(qlinear_mfma_wide_kernel, dim3(ids), dim3(512), KW::LDS, st, a, blocks, row_blocks, S);
   return check_launch();
 }
 
@@ -1292,7 +1326,7 @@ int qlinear_num_lora_splits(int K, int N);
 int qlinear_num_splits(int K, int N, int M) {
   if (M > 128) {
     // 256-row blocks: K-slices only while the launch has fewer workgroups than CUs
-    const int wgs = (N + 127) / 128 * ((M + 255) / 256);
+    const int wgs = (N + 255) / 256 * ((M + 255) / 256);
     int s = 1;
     while (wgs * s < 192 && s * 2 <= TMX_MAX_SPLITS && slices_ok(K / 64, s * 2) && slice_len(K / 64, s * 2) >= 8) s *= 2;
     return s;

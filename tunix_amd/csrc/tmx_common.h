@@ -66,6 +66,17 @@ __device__ __forceinline__ int acc_row(int r, int lane) {
   return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
 }
 
+// The same expansion in four parts, for loops that spread the dequantisation between MFMAs:
+// dequant_masks() once per word, then register p of the B operand (elements 2p, 2p + 1 =
+// nibbles p, p + 4) from dequant_part<p>().  Bit-identical to dequant_word().
+__device__ __forceinline__ void dequant_masks(uint32_t d, uint32_t& lo, uint32_t& hi) {
+  lo = d & 0x0F0F0F0Fu;
+  hi = (d >> 4) & 0x0F0F0F0Fu;
+  asm volatile("" : "+v"(lo), "+v"(hi));
+}
+template <int P>
+__device__ __forceinline__ uint32_t dequant_part(uint32_t lo, uint32_t hi, float s, float m8s);
+
 // Expand one 32-bit word (8 nibbles, element j = 2 (i % 4) + i / 4 for nibble i)
 // into the 8 bf16 B-operand values of one MFMA step: bf16((u - 8) * s).
 __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s) {
@@ -88,6 +99,13 @@ __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s)
   bf16x8_t b;
   __builtin_memcpy(&b, p, 16);
   return b;
+}
+
+template <int P>
+__device__ __forceinline__ uint32_t dequant_part(uint32_t lo, uint32_t hi, float s, float m8s) {
+  const uint32_t w = (P & 1) ? hi : lo;  // nibbles P and P + 4: bytes P / 2 and P / 2 + 2 of that word
+  const float a = (float)((w >> (8 * (P / 2))) & 0xFF), b = (float)((w >> (8 * (P / 2) + 16)) & 0xFF);
+  return pack_bf2(fmaf(a, s, m8s), fmaf(b, s, m8s));
 }
 
 
