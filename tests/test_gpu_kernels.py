@@ -194,22 +194,27 @@ def test_rope_kv_write(family, H, N, Kh):
   assert np.all(kc_h[:, others] == 7.0) and np.all(vc_h[:, others] == 7.0)
 
 
-@pytest.mark.parametrize('M,F,ns', [(3, 1024, 0), (64, 14336, 2), (5, 768, 1)])
-def test_swiglu(M, F, ns):
+@pytest.mark.parametrize('M,F,ns,lora', [
+    (3, 1024, 0, False), (64, 14336, 2, True), (5, 768, 1, True), (5, 768, 0, True),
+    # more than 128 rows of bf16 input: 16 rows per workgroup, ragged last block and column tail
+    (300, 2304, 0, True), (200, 1024, 0, False), (129, 4096, 0, True),
+])
+def test_swiglu(M, F, ns, lora):
   T = G.Keep()
-  rng = np.random.default_rng(F)
+  rng = np.random.default_rng(F + M)
   r = 16
   lb = bf16_round(rng.standard_normal((r, 2 * F)).astype(np.float32) * 0.05)
   act = torch.empty(M, F, dtype=torch.bfloat16, device=G.DEV)
+  tp = rng.standard_normal((28, M, 128)).astype(np.float32)
+  lora_args = (T.f32(tp), 28, 128, T.bf(lb), r, 2.0) if lora else (None, 0, 0, None, 0, 0.0)
   if ns == 0:
-    gu = bf16_round(rng.standard_normal((M, 2 * F)).astype(np.float32) * 2)
-    G.call('tmx_swiglu', S(), T.bf(gu), None, 0, None, 0, 0, None, 0, 0.0, G.p(act), M, F)
-    y = gu
+    y = bf16_round(rng.standard_normal((M, 2 * F)).astype(np.float32) * 2)
+    G.call('tmx_swiglu', S(), T.bf(y), None, 0, *lora_args, G.p(act), M, F)
   else:
     gp = rng.standard_normal((ns, M, 2 * F)).astype(np.float32)
-    tp = rng.standard_normal((28, M, 128)).astype(np.float32)
-    G.call('tmx_swiglu', S(), None, T.f32(gp), ns, T.f32(tp), 28, 128, T.bf(lb), r, 2.0, G.p(act), M, F)
+    G.call('tmx_swiglu', S(), None, T.f32(gp), ns, *lora_args, G.p(act), M, F)
     y = bf16_round(gp.sum(0))
+  if lora:
     t = bf16_round(tp.sum(0))
     dg = bf16_round(bf16_round(t[:, :r] @ lb[:, :F]) * np.float32(2.0))
     du = bf16_round(bf16_round(t[:, r:2 * r] @ lb[:, F:]) * np.float32(2.0))

@@ -452,8 +452,95 @@ __global__ __launch_bounds__(256) void swiglu_kernel(SwigluArgs a) {
   *reinterpret_cast<uint4*>(a.act + (size_t)m * a.F + f0) = pack8(o);
 }
 
+// Many rows (cache fill): grid (ceil(F / 2048), ceil(M / 16)); a thread owns 8 adjacent hidden
+// units of 16 rows.  Its columns of B (gate and up, rank <= 16) stay in registers for all 16 rows,
+// packed as bf16 pairs along the rank, and the rank sum runs on the packed bf16 dot product
+// (two products and the add per instruction; t is bf16 already, so the products are exact and
+// only the f32 summation order differs from the one-row kernel).  bf16 input only.
+constexpr int kSwigluRows = 16;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_of(const uint4& v, int e) {
+  const uint32_t w = e < 2 ? v.x : (e < 4 ? v.y : (e < 6 ? v.z : v.w));
+  return (e & 1) ? (w >> 16) : (w & 0xFFFFu);
+}
+__global__ __launch_bounds__(256) void swiglu_rows_kernel(SwigluArgs a, int M) {
+  __shared__ uint32_t t_s[kSwigluRows][16];  // [row][gate pairs 0..7 | up pairs 0..7]
+  const int m0 = blockIdx.y * kSwigluRows;
+  const int rows = M - m0 < kSwigluRows ? M - m0 : kSwigluRows;
+  const int f0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const bool mine = f0 < a.F;
+  const int r = a.lora.t_part ? a.lora.r : 0;
+  uint32_t pg[8][8], pu[8][8];  // [rank pair][column]: (B[2p][c], B[2p + 1][c])
+  if (mine && r) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const uint4 z = {0, 0, 0, 0};
+      const uint16_t* b0 = a.lora.b + (size_t)(2 * p) * 2 * a.F + f0;
+      const uint16_t* b1 = b0 + 2 * a.F;
+      const uint4 g0 = 2 * p < r ? *reinterpret_cast<const uint4*>(b0) : z;
+      const uint4 g1 = 2 * p + 1 < r ? *reinterpret_cast<const uint4*>(b1) : z;
+      const uint4 u0 = 2 * p < r ? *reinterpret_cast<const uint4*>(b0 + a.F) : z;
+      const uint4 u1 = 2 * p + 1 < r ? *reinterpret_cast<const uint4*>(b1 + a.F) : z;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pg[p][e] = bf16_of(g0, e) | (bf16_of(g1, e) << 16);
+        pu[p][e] = bf16_of(u0, e) | (bf16_of(u1, e) << 16);
+      }
+    }
+  }
+  // t pairs: bf16(sum of the planes' values) of columns x.A_gate | x.A_up, zero past the rank
+  if (r) {
+    const int row = threadIdx.x >> 4, c = threadIdx.x & 15, half = c >> 3, p = c & 7;
+    float t0 = 0.f, t1 = 0.f;
+    if (row < rows) {
+      const float* q = a.lora.t_part + (size_t)(m0 + row) * a.lora.ldt + half * r + 2 * p;
+      for (int sp = 0; sp < a.lora.nsplit; ++sp) {
+        if (2 * p < r) t0 += q[(size_t)sp * M * a.lora.ldt];
+        if (2 * p + 1 < r) t1 += q[(size_t)sp * M * a.lora.ldt + 1];
+      }
+    }
+    t_s[row][c] = pack_bf2(t0, t1);
+  }
+  __syncthreads();
+  if (!mine) return;
+  for (int i = 0; i < rows; ++i) {
+    const size_t m = m0 + i;
+    float g[8], u[8], o[8];
+    unpack8(*reinterpret_cast<const uint4*>(a.gu_bf16 + m * 2 * a.F + f0), g);
+    unpack8(*reinterpret_cast<const uint4*>(a.gu_bf16 + m * 2 * a.F + a.F + f0), u);
+    if (r) {
+      float dg[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, du[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const bf16x2_t tg = __builtin_bit_cast(bf16x2_t, t_s[i][p]), tu = __builtin_bit_cast(bf16x2_t, t_s[i][8 + p]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          dg[e] = __builtin_amdgcn_fdot2_f32_bf16(tg, __builtin_bit_cast(bf16x2_t, pg[p][e]), dg[e], false);
+          du[e] = __builtin_amdgcn_fdot2_f32_bf16(tu, __builtin_bit_cast(bf16x2_t, pu[p][e]), du[e], false);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        g[e] = rbf(g[e] + rbf(rbf(dg[e]) * a.lora.ls));
+        u[e] = rbf(u[e] + rbf(rbf(du[e]) * a.lora.ls));
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float sg = rbf(1.f / (1.f + expf(-g[e])));
+      o[e] = rbf(g[e] * sg) * u[e];
+    }
+    *reinterpret_cast<uint4*>(a.act + m * a.F + f0) = pack8(o);
+  }
+}
+
 int swiglu(hipStream_t st, const SwigluArgs& a, int M) {
   if (a.F % 8 || (a.lora.t_part && 2 * a.lora.r > TMX_MAX_RPAD)) return TMX_ERR_SHAPE;
+  if (M > 128 && a.gu_bf16 && (!a.lora.t_part || a.lora.r <= 16)) {
+    hipLaunchKernelGGL(swiglu_rows_kernel, dim3((a.F + 2047) / 2048, (M + kSwigluRows - 1) / kSwigluRows), dim3(256),
+                       0, st, a, M);
+    return check_launch();
+  }
   hipLaunchKernelGGL(swiglu_kernel, dim3((a.F + 2047) / 2048, M), dim3(256), 0, st, a);
   return check_launch();
 }

@@ -222,7 +222,7 @@ class Sampler:
     return s
 
   MAX_ROWS = 128        # rows of one pass with the head (sequences x tokens per pass)
-  MAX_FILL_ROWS = 2048  # rows of one cache-fill pass of a dense model (256-row projection blocks)
+  MAX_FILL_ROWS = 4096  # rows of one cache-fill pass of a dense model (256-row projection blocks)
 
   def _fill_rows(self):
     cfg = self._transformer.config
