@@ -344,6 +344,41 @@ def main():
         result['roofline_all'][n] = {'avg_launch_ms': avg, 'achieved_GBps': alg[n] / (avg * 1e-3) / 1e9,
                                      'frac': alg[n] / (avg * 1e-3) / 8e12}
 
+  if not args.no_profile and not cfg.num_experts and sampler._fill_rows() > 128:
+    # Cache fill (outside the headline metric): the prompt walk above, and the projection kernel that
+    # carries it (256-row blocks, MFMA-bound) timed alone on the gate|up shape at the rows of one pass.
+    lib = _lib.lib()
+    rows = min(sampler._fill_rows() // batch, 128, prompt - 1) * batch
+    pl = model.layers[0]['gate_up']
+    xs = torch.randn(rows, pl.k, device='cuda').to(torch.bfloat16)
+    ns = lib.tmx_qlora_linear_num_splits(rows, pl.k, pl.n)
+    yp = torch.empty(ns, rows, pl.n, dtype=torch.float32, device='cuda')
+    tp = torch.empty(32, rows, 128, dtype=torch.float32, device='cuda')
+    a_t = pl.lora_a_t.data_ptr() if pl.lora_a_t is not None else None
+    def gemm():
+      _lib.check(lib.tmx_qlora_linear_planes(_lib.stream(), xs.data_ptr(), pl.qweight.data_ptr(), pl.scales.data_ptr(),
+                                             a_t, yp.data_ptr(), tp.data_ptr(), rows, pl.k, pl.n, group,
+                                             pl.r_pad if a_t else 0, ns), 'tmx_qlora_linear_planes')
+    for _ in range(2):
+      gemm()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(8):
+      gemm()
+    e1.record()
+    torch.cuda.synchronize()
+    g_ms = e0.elapsed_time(e1) / 8
+    flops = 2.0 * rows * pl.k * pl.n
+    result['prefill'] = {
+        'prompt_tokens_per_s': batch * (prompt - 1) / (walk_ms[0] * 1e-3), 'walk_ms': walk_ms[0],
+        'rows_per_pass': rows,
+        'roofline': {'bound': 'mfma', 'kernel': 'tmx::qlinear_mfma_wide_kernel',
+                     'shape': f'{rows} x {pl.k} x {pl.n} (gate|up)', 'avg_launch_ms': g_ms,
+                     'achieved': flops / (g_ms * 1e-3) / 1e12, 'peak': 2500.0, 'unit': 'TFLOP/s',
+                     'frac': flops / (g_ms * 1e-3) / 2.5e15},
+    }
+    del xs, yp, tp
+
   if not args.no_cpu_baseline and not cfg.num_experts:
     del st
     result['cpu_baseline'] = cpu_baseline(args.workload)
