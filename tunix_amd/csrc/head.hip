@@ -135,8 +135,9 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
   for (int m = 0; m < MT; ++m) {
     const int row = m * 32 + nl;
     const int tpp = a.tpp > 0 ? a.tpp : 1;
+    const int prow = a.row_base + row;  // row of the pass
     target[m] = (score && row < a.M)
-                    ? a.token_buffer[(size_t)(row / tpp) * a.buf_len + *a.step + row % tpp + 1] : -1;
+                    ? a.token_buffer[(size_t)(prow / tpp) * a.buf_len + *a.step + prow % tpp + 1] : -1;
   }
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
@@ -251,8 +252,9 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
     }
     if (a.mode == TMX_SAMPLE_SCORE) {  // teacher forcing: the token stays, only its log-prob is written
       const int tpp = a.tpp > 0 ? a.tpp : 1;
+      const int prow = a.row_base + row;
       if (a.logprobs)
-        a.logprobs[(size_t)(row / tpp) * a.buf_len + *a.step + row % tpp + 1] = (best.z - mx) - logf(se);
+        a.logprobs[(size_t)(prow / tpp) * a.buf_len + *a.step + prow % tpp + 1] = (best.z - mx) - logf(se);
       return;
     }
     const int col = *a.step + 1;

@@ -153,6 +153,7 @@ struct HeadArgs {
   int n_eos;
   int buf_len;
   int tpp;  // tokens per pass (0: 1), score mode only: row m is sequence m / tpp at column *step + m % tpp
+  int row_base;  // score mode: x holds rows row_base .. row_base + M - 1 of the pass (chunks of <= 128 rows)
 };
 
 

@@ -221,8 +221,8 @@ class Sampler:
       s.nucleus_workspace, s.nucleus_workspace_bytes = self._nucleus_ws.data_ptr(), self._nucleus_ws.numel()
     return s
 
-  MAX_ROWS = 128        # rows of one pass with the head (sequences x tokens per pass)
-  MAX_FILL_ROWS = 4096  # rows of one cache-fill pass of a dense model (256-row projection blocks)
+  MAX_ROWS = 128        # rows of one pass that chooses tokens (sequences x tokens per pass)
+  MAX_FILL_ROWS = 4096  # rows of one cache-fill or scoring pass of a dense model (256-row projection blocks)
 
   def _fill_rows(self):
     cfg = self._transformer.config
@@ -236,7 +236,9 @@ class Sampler:
     MAX_ROWS rows (MAX_FILL_ROWS without the head, where the model allows), instead of one
     token per launch sequence."""
     b = st['token_buffer'].shape[0]
-    per = min(128, max(1, (self.MAX_ROWS if sample else self._fill_rows()) // b))
+    # the head chooses tokens for up to MAX_ROWS rows; scoring takes as many rows as a cache fill
+    choose = sample and st['sampling_mode'] != 'score'
+    per = min(128, max(1, (self.MAX_ROWS if choose else self._fill_rows()) // b))
     while n_tokens > 0:
       t = min(per, n_tokens)
       self.run_steps(st, 1, sample=sample, tokens_per_pass=t)
