@@ -267,6 +267,165 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Scoring passes with many rows (teacher forcing over whole sequences): the same product as a
+// matrix-pipe-bound kernel.  A workgroup multiplies 256 vocabulary rows by 256 sequence rows:
+// the vocabulary rows are the A operand and come through a double-buffered LDS slab filled by
+// direct-to-LDS loads (256-byte rows of a 128-wide k-step, chunks XOR-swizzled by row % 16);
+// wave w owns sequence rows 32 w .. 32 w + 31 as the B operand, read straight from global
+// memory, 64 contiguous bytes per lane and k-tile (lane (row, h) holds k = 32 h .. 32 h + 31 of
+// the tile, MFMA step t pairs k = 32 h + 8 t .. with the same k of the vocabulary rows).  A lane's
+// 128 accumulator registers are 128 vocabulary rows of ONE sequence row, so max / sum-exp / the
+// target's z run down the registers.  LDS reads of fragment group g + 1 and the refill of the
+// B registers are pinned between the MFMAs of group g.  Consecutive workgroups take the
+// sequence-row blocks of one vocabulary block, so the head matrix leaves HBM once.
+struct HW {
+  static constexpr int MT = 8, ROWS = 256, TS = 2, XS = 128;
+  static constexpr size_t LDS = (size_t)2 * ROWS * XS * 2;  // 128 KiB
+};
+
+__global__ __launch_bounds__(512, 1) void head_score_wide_kernel(HeadArgs a, int tok_blocks, int voc_blocks) {
+  extern __shared__ __align__(16) uint16_t smem[];
+  constexpr int MT = HW::MT, TS = HW::TS, XS = HW::XS, ROWS = HW::ROWS;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, nl = lane & 31;
+  const int vb = (int)blockIdx.x / tok_blocks, tb = (int)blockIdx.x % tok_blocks;
+  if (vb >= voc_blocks) return;
+  const int v0 = vb * ROWS;
+  const int vrows = a.V - v0 < ROWS ? a.V - v0 : ROWS;
+  const int tok = tb * 256 + wave * 32 + nl;       // sequence row of this lane's accumulator column
+  const int tok_l = tok < a.M ? tok : a.M - 1;
+  const int nsteps = a.D >> 7, last_step = nsteps - 1;
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.w + (size_t)v0 * a.D, (uint32_t)vrows * a.D * 2u);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, (uint32_t)a.M * a.D * 2u);
+  constexpr int XR = ROWS / 32;
+  int woff[XR];  // slab transfer: load i moves vocabulary rows 4 wave + 32 i .. + 3, 16 lanes each
+#pragma unroll
+  for (int i = 0; i < XR; ++i) {
+    const int row_l = 4 * wave + 32 * i + (lane >> 4);
+    woff[i] = (row_l < vrows ? row_l : vrows - 1) * a.D * 2 + (((lane & 15) ^ (row_l & 15)) * 16);
+  }
+  const int xv = tok_l * a.D * 2 + h * 64;
+
+  f32x16_t acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
+  u32x4_t breg[4 * TS];  // B fragments of the 8 groups of a step, refilled for the next step after use
+
+  auto load_b = [&](int step, auto gc) __attribute__((always_inline)) {
+    constexpr int g = decltype(gc)::value;
+    step = step < last_step ? step : last_step;
+    breg[g] = __builtin_amdgcn_raw_buffer_load_b128(rx, xv + (g & 3) * 16, (step * TS + (g >> 2)) * 128, 0);
+  };
+  auto dma_w = [&](int step, int buf) __attribute__((always_inline)) {
+    step = step < last_step ? step : last_step;
+    uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * 4 * XS;
+#pragma unroll
+    for (int i = 0; i < XR; ++i) load_row_to_lds(rw, base + i * 32 * XS, woff[i], step * (TS * 128));
+  };
+  constexpr int kYounger = 4 * TS;
+  auto wait_slab = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
+    __syncthreads();
+  };
+  auto step_math = [&](int step, int buf) __attribute__((always_inline)) {
+    const uint16_t* wb = smem + (size_t)buf * ROWS * XS + nl * XS;
+    bf16x8_t wq[2][MT];
+    {
+      // group g = 4 j + t needs k = 64 j + 32 h + 8 t ..: chunk 8 j + 4 h + t of the slab row
+      const int slot = ((4 * h) ^ (nl & 15)) * 8;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) wq[0][m] = *reinterpret_cast<const bf16x8_t*>(wb + m * 32 * XS + slot);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<4 * TS>([&](auto gc) __attribute__((always_inline)) {
+      constexpr int g = decltype(gc)::value, cur = g & 1, nxt = cur ^ 1;
+      constexpr bool more = g + 1 < 4 * TS;
+      constexpr int gn = g + 1;
+      const int slot = ((8 * (gn >> 2) + 4 * h + (gn & 3)) ^ (nl & 15)) * 8;
+      const bf16x8_t b = __builtin_bit_cast(bf16x8_t, breg[g]);
+      static_for<MT>([&](auto mc) __attribute__((always_inline)) {
+        constexpr int m = decltype(mc)::value;
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wq[cur][m], b, acc[m], 0, 0, 0);
+        if constexpr (more) {
+          wq[nxt][m] = *reinterpret_cast<const bf16x8_t*>(wb + m * 32 * XS + slot);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+      load_b(step + 1, gc);  // fragment consumed: refill it for the next step
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  dma_w(0, 0);
+  static_for<4 * TS>([&](auto gc) __attribute__((always_inline)) { load_b(0, gc); });
+  wait_slab();
+  for (int step = 0; step < nsteps; ++step) {
+    const int buf = step & 1;
+    dma_w(step + 1, buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    step_math(step, buf);
+    wait_slab();
+  }
+
+  // per sequence row: running max and sum of exp over this block's vocabulary rows, and the z of
+  // the given next token if it lies in the block (key 0 marks it, as in head_kernel's score mode)
+  const int tpp = a.tpp > 0 ? a.tpp : 1;
+  const int target = a.token_buffer[(size_t)(tok_l / tpp) * a.buf_len + *a.step + tok_l % tpp + 1];
+  float mx = kNegBig, se = 0.f;
+  Best best = {-INFINITY, -INFINITY, 0x7FFFFFFF};
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int v = v0 + m * 32 + acc_row(r, lane);
+      if (v >= a.V) continue;
+      const float z = rbf(acc[m][r]) / a.temperature;
+      if (z > mx) {
+        se = se * expf(mx - z) + 1.f;
+        mx = z;
+      } else {
+        se += expf(z - mx);
+      }
+      if (v == target) best = {0.f, z, v};
+    }
+  {
+    const float mx2 = __shfl_xor(mx, 32, 64), se2 = __shfl_xor(se, 32, 64);
+    Best o = {__shfl_xor(best.key, 32, 64), __shfl_xor(best.z, 32, 64), __shfl_xor(best.idx, 32, 64)};
+    lse_merge(mx, se, mx2, se2);
+    best_merge(best, o);
+  }
+  if (h == 0 && tok < a.M) {
+    float* pf = a.part_f + ((size_t)tok * a.nwg + vb) * 4;
+    pf[0] = mx; pf[1] = se; pf[2] = best.key; pf[3] = best.z;
+    a.part_i[(size_t)tok * a.nwg + vb] = best.idx;
+  }
+}
+
+// Scoring of M rows (any count) with the wide kernel + the finalize kernel; the caller has checked
+// mode == TMX_SAMPLE_SCORE, no forbidden ids, no logits output, D % 128 == 0.
+int head_score_wide(hipStream_t st, HeadArgs a) {
+  if (a.D % 128 || a.M <= 0 || (size_t)a.M * a.D * 2 >= (1u << 31) || (size_t)256 * a.D * 2 >= (1u << 31))
+    return TMX_ERR_SHAPE;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&head_score_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)HW::LDS);
+  if (attr != hipSuccess) return TMX_ERR_LAUNCH;
+  const int tok_blocks = (a.M + 255) / 256, voc_blocks = (a.V + HW::ROWS - 1) / HW::ROWS;
+  a.nwg = voc_blocks;
+  a.row_base = 0;
+  hipLaunchKernelGGL(head_score_wide_kernel, dim3(tok_blocks * voc_blocks), dim3(512), HW::LDS, st, a, tok_blocks,
+                     voc_blocks);
+  int rc = check_launch();
+  if (rc != TMX_OK) return rc;
+  hipLaunchKernelGGL(head_finalize_kernel, dim3(a.M), dim3(256), 0, st, a);
+  return check_launch();
+}
+
 int head_logits(hipStream_t st, HeadArgs& a) {
   if (a.V % 32 || a.D % 64 || a.M <= 0 || a.M > 128) return TMX_ERR_SHAPE;
   a.nwg = (a.V + 127) / 128;
