@@ -147,6 +147,17 @@ int tmx_gqa_decode_attention(void* stream, const void* q, const void* kcache, co
                              const uint8_t* input_mask, const int32_t* step, int buf_len, void* out,
                              void* workspace, int B, int N, int Kh, int H, int C);
 
+/* The same for T consecutive query tokens of every sequence (cache fill and scoring passes):
+ * q and out are [n_seq * T, N H], row s * T + t is the token at slot *step + t of sequence s and
+ * attends to the slots j <= *step + t with input_mask[s, j] (the causal mask of
+ * tunix/generate/utils.py:2116-2229 restricted to the rows of the pass); K and V of the pass's
+ * own tokens must already be in the caches.  From 4 tokens per sequence on, a workgroup walks the
+ * cache once for a block of tokens (MFMA kernel, head_dim 64 or 128); below, every row runs the
+ * decode kernel.  workspace: tmx_gqa_decode_workspace_bytes(n_seq * T, N, Kh, H, C) bytes. */
+int tmx_gqa_attention_rows(void* stream, const void* q, const void* kcache, const void* vcache,
+                           const uint8_t* input_mask, const int32_t* step, int buf_len, void* out,
+                           void* workspace, int n_seq, int T, int N, int Kh, int H, int C);
+
 /* ---- final projection + log-softmax + token selection ---------------------- */
 
 /* logits = bf16(x[M, D] . head_w[V, D]^T) as f32; forbidden ids -> -inf; mode

@@ -296,6 +296,40 @@ def test_gqa_decode_attention(B, N, Kh, H, C, step):
   assert np.abs(got - ref).max() < 2e-2
 
 
+@pytest.mark.parametrize('nseq,T,N,Kh,H,C,step', [
+    (2, 40, 4, 4, 64, 64, 3), (3, 9, 8, 2, 64, 96, 50), (2, 33, 32, 8, 128, 300, 200), (1, 64, 8, 1, 128, 128, 0),
+    (2, 5, 16, 8, 128, 96, 60), (1, 128, 4, 4, 128, 200, 31), (2, 3, 8, 4, 64, 64, 20),
+])
+def test_gqa_attention_rows(nseq, T, N, Kh, H, C, step):
+  """T consecutive query tokens per sequence against the per-token oracle (row t sees slots <= step + t)."""
+  Tk = G.Keep()
+  rng = np.random.default_rng(nseq * 1000 + C + T)
+  q = bf16_round(rng.standard_normal((nseq, T, N, H)).astype(np.float32))
+  k = bf16_round(rng.standard_normal((nseq, C, Kh, H)).astype(np.float32))
+  v = bf16_round(rng.standard_normal((nseq, C, Kh, H)).astype(np.float32))
+  in_mask = np.ones((nseq, C), bool)
+  for b in range(nseq):  # left padding of different lengths plus a hole
+    in_mask[b, : (b * 5 + 2) % max(step, 1)] = False
+  in_mask[0, (step + T) // 2] = False
+  in_mask[:, step] = True
+  lib = _lib.lib()
+  ws = torch.empty(max(lib.tmx_gqa_decode_workspace_bytes(nseq * T, N, Kh, H, C), 4), dtype=torch.uint8, device=G.DEV)
+  out = torch.empty(nseq * T, N * H, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_gqa_attention_rows', S(), Tk.bf(q.reshape(nseq * T, N * H)), Tk.bf(k), Tk.bf(v), Tk.u8(in_mask),
+         Tk.i32([step]), C, G.p(out), G.p(ws), nseq, T, N, Kh, H, C)
+  G.sync()
+  from oracle import masks as OMK
+  got = G.host(out).reshape(nseq, T, N * H)
+  for t in range(T):
+    mask = OMK.compute_attention_masks(step + t, C, ~in_mask)
+    fused = L.gqa_attention(q[:, t:t + 1], k, v, mask, BF16, 'fused').reshape(nseq, -1)
+    ref = L.gqa_attention(q[:, t:t + 1], k, v, mask, BF16, 'reference').reshape(nseq, -1)
+    # as the one-token kernel: 1 ulp against the f32-internal oracle, bf16 noise against the
+    # reference-rounding oracle
+    G.assert_bf16_close(got[:, t], fused, ulps=1.0, extra=1e-3, what=f'attention rows, token {t}')
+    assert np.abs(got[:, t] - ref).max() < 2e-2, (t, np.abs(got[:, t] - ref).max())
+
+
 def _head_inputs(M, D, V, seed):
   rng = np.random.default_rng(seed)
   x = bf16_round(rng.standard_normal((M, D)).astype(np.float32))

@@ -351,7 +351,9 @@ def test_per_token_logps_match_oracle_and_the_rollout_logprobs():
                                       eos_tokens=[-1], return_logprobs=True, seed=3), prompt_token_ids=prompts)
   gen = np.stack(ro.tokens)
   scored = r.get_per_token_logps(ro.left_padded_prompt_tokens, gen)
-  np.testing.assert_allclose(scored, np.stack(ro.logprobs), atol=2e-5)
+  # the scoring pass walks several tokens per sequence through the many-token attention kernel, the
+  # rollout decoded them one by one: same values up to bf16 rounding flips of the hidden states
+  assert np.abs(scored - np.stack(ro.logprobs)).max() <= LOGPROB_TOL
   with pytest.raises(ValueError):
     s.per_token_logps(np.zeros((2, 0), np.int32), comp[:2])
 

@@ -27,6 +27,7 @@ SIGNATURES = {
     'tmx_swiglu': [vp, vp, vp, ci, vp, ci, ci, vp, ci, cf, vp, ci, ci],
     'tmx_qlora_gate_up_swiglu': [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cf],
     'tmx_gqa_decode_attention': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci],
+    'tmx_gqa_attention_rows': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci, ci],
     'tmx_head_sample': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
                         vp, vp],
     'tmx_head_sample_nucleus': [vp, vp, vp, ci, ci, ci, cf, cf, ci, cu32, cu32, vp, vp, ci, vp, ci, vp, vp,

@@ -190,6 +190,180 @@ __global__ __launch_bounds__(H) void gqa_combine_kernel(AttnArgs a) {
   a.out[((size_t)b * a.N + kvh * G + g) * H + d] = f2bf(ls > 0.f ? o / ls : 0.f);
 }
 
+// ---------------------------------------------------------------------------
+// Many tokens per sequence (cache fill and scoring passes): a workgroup owns one (sequence, kv
+// head) and a block of consecutive query tokens, and walks the cache once for all of them, 32
+// positions at a time, on the matrix pipe.  Wave w holds 32 query rows (32 / G tokens x G heads)
+// as the B operand; the K tile [32 positions, H] and the V tile go global -> LDS by direct loads
+// (16-byte chunks XOR-swizzled by row) and are shared by the four waves.
+//   scores^T [position, query] = K . Q^T : lane (query, h) keeps 16 positions of ONE query in its
+//     accumulator, so mask, max, exp and sum run down the registers (one shuffle joins the halves);
+//   out^T [hidden, query] += V^T . P^T  : the B operand is the lane's own 8 probabilities of a
+//     16-position block (positions are consumed in accumulator order, which V^T follows: its
+//     fragment is gathered from the V tile with 16-bit LDS reads), and the rescale by
+//     exp(old max - new max) is per lane.
+// Probabilities enter the product as two bf16 terms (hi + lo), i.e. with 16 mantissa bits.
+constexpr int kFillMinTokens = 4;  // tokens per sequence and pass from which the fill kernel is used
+
+template <int H, int G>
+__global__ __launch_bounds__(256) void gqa_fill_kernel(AttnArgs a) {
+  constexpr int KS = H / 16;        // MFMA k-steps of the score product
+  constexpr int CPR = H / 8;        // 16-byte chunks per cache row
+  constexpr int RPD = 64 / CPR;     // rows per 1 KiB direct-to-LDS load
+  constexpr int NLD = 32 / RPD / 4; // loads per wave and tile
+  constexpr int HT = H / 32;        // hidden tiles of the output
+  constexpr int TPW = 32 / G, TQ = 4 * TPW;  // tokens per wave / workgroup
+  __shared__ __align__(16) uint16_t kt[2][32 * H], vt[2][32 * H];
+  const int kvh = blockIdx.x, seq = blockIdx.y, tblk = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int h = lane >> 5, qi = lane & 31;
+  const int T = a.tpp, step0 = *a.step;
+  const int tok = tblk * TQ + wave * TPW + qi / G, g = qi % G;
+  const int tok_l = tok < T ? tok : T - 1;
+  const int limit = step0 + tok_l;  // newest slot this query sees
+  const int last_tok = tblk * TQ + TQ - 1 < T - 1 ? tblk * TQ + TQ - 1 : T - 1;
+  const int nblk = (step0 + last_tok + 32) >> 5;  // blocks of 32 positions up to the newest slot of the block
+
+  const size_t qoff = ((size_t)(seq * T + tok_l) * a.N + kvh * G + g) * H;
+  u32x4_t qf[KS];
+#pragma unroll
+  for (int t = 0; t < KS; ++t) qf[t] = *reinterpret_cast<const u32x4_t*>(a.q + qoff + (H / 2) * h + 8 * t);
+
+  const uint32_t row_bytes = (uint32_t)a.Kh * H * 2;
+  const uint32_t span = ((uint32_t)(a.C - 1) * a.Kh + 1) * H * 2;  // rows past the cache read zero
+  const __amdgpu_buffer_rsrc_t rk = make_rsrc(a.kcache + ((size_t)seq * a.C * a.Kh + kvh) * H, span);
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(a.vcache + ((size_t)seq * a.C * a.Kh + kvh) * H, span);
+  int toff[NLD];  // tile transfer: load i of this wave moves rows (wave + 4 i) RPD .. + RPD - 1
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    const int row_l = (wave + 4 * i) * RPD + lane / CPR;
+    toff[i] = row_l * row_bytes + (((lane % CPR) ^ (row_l % CPR)) * 16);
+  }
+  auto dma_tile = [&](int blk, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      load_row_to_lds(rk, &kt[buf][(wave + 4 * i) * RPD * H], toff[i], blk * 32 * row_bytes);
+      load_row_to_lds(rv, &vt[buf][(wave + 4 * i) * RPD * H], toff[i], blk * 32 * row_bytes);
+    }
+  };
+  // input mask of a block: lane p of the lower half fetches the byte of position 32 blk + p early,
+  // the ballot that turns the bytes into a bit per position runs when the block is needed
+  const uint8_t* mrow = a.input_mask + (size_t)seq * a.buf_len;
+  auto mask_byte = [&](int blk) __attribute__((always_inline)) {
+    const int p = blk * 32 + qi;
+    return (h == 0 && p < a.buf_len) ? mrow[p] : (uint8_t)0;
+  };
+  f32x16_t o[HT];
+#pragma unroll
+  for (int c = 0; c < HT; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[c][r] = 0.f;
+  float m = -1e30f, l = 0.f;
+
+  uint8_t mb = mask_byte(0);
+  dma_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  for (int blk = 0; blk < nblk; ++blk) {
+    const int buf = blk & 1;
+    const uint32_t mbits = (uint32_t)__ballot(mb != 0);
+    mb = mask_byte(blk + 1);  // requested before the tile so that the tile's loads stay the youngest
+    if (blk + 1 < nblk) dma_tile(blk + 1, buf ^ 1);
+    // scores^T: rows = positions of the block, column = this lane's query
+    f32x16_t sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    const uint16_t* kb = &kt[buf][qi * H];
+#pragma unroll
+    for (int t = 0; t < KS; ++t) {
+      const int slot = ((KS * h + t) ^ (qi % CPR)) * 8;  // lane (position, h) multiplies k = (H / 2) h + 8 t ..
+      const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kb + slot);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, __builtin_bit_cast(bf16x8_t, qf[t]), sacc, 0, 0, 0);
+    }
+    float sc[16];
+    float mn = m;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int pl = acc_row(r, lane), p = blk * 32 + pl;
+      const bool ok = p <= limit && ((mbits >> pl) & 1u);
+      sc[r] = ok ? sacc[r] * a.scale : -1e30f;
+      mn = fmaxf(mn, sc[r]);
+    }
+    mn = fmaxf(mn, __shfl_xor(mn, 32, 64));
+    const float alpha = __expf(m - mn);
+    m = mn;
+    // probabilities as bf16 pairs hi + lo (16 mantissa bits between them), so that the product
+    // keeps the precision of the one-token kernel's f32 probabilities and a scoring pass
+    // reproduces the log-probs of the rollout that generated the tokens
+    float ps = 0.f;
+    uint32_t pk[8], pl2[8];
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      const float p0 = sc[r] > -1e29f ? __expf(sc[r] - mn) : 0.f;
+      const float p1 = sc[r + 1] > -1e29f ? __expf(sc[r + 1] - mn) : 0.f;
+      pk[r >> 1] = pack_bf2(p0, p1);
+      pl2[r >> 1] = pack_bf2(p0 - bf_lo(pk[r >> 1]), p1 - bf_hi(pk[r >> 1]));
+      ps += p0 + p1;
+    }
+    l = l * alpha + ps;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int c = 0; c < HT; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[c][r] *= alpha;
+    }
+    // out^T += V^T . P^T, 16 positions (accumulator registers 8 kb .. 8 kb + 7) per MFMA
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; ++kb2) {
+      const u32x4_t pf = {pk[4 * kb2], pk[4 * kb2 + 1], pk[4 * kb2 + 2], pk[4 * kb2 + 3]};
+      const u32x4_t pg = {pl2[4 * kb2], pl2[4 * kb2 + 1], pl2[4 * kb2 + 2], pl2[4 * kb2 + 3]};
+#pragma unroll
+      for (int c = 0; c < HT; ++c) {
+        uint32_t vw[4];
+#pragma unroll
+        for (int j2 = 0; j2 < 4; ++j2) {
+          uint32_t e2[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const int j = 2 * j2 + e;
+            const int row = (2 * kb2 + j / 4) * 8 + 4 * h + (j & 3);  // = acc_row(8 kb2 + j, lane)
+            const int chunk = 4 * c + (qi >> 3);
+            e2[e] = vt[buf][row * H + ((chunk ^ (row % CPR)) * 8) + (qi & 7)];
+          }
+          vw[j2] = e2[0] | (e2[1] << 16);
+        }
+        const u32x4_t vf = {vw[0], vw[1], vw[2], vw[3]};
+        o[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                       __builtin_bit_cast(bf16x8_t, pf), o[c], 0, 0, 0);
+        o[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                       __builtin_bit_cast(bf16x8_t, pg), o[c], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile has landed
+    __syncthreads();
+  }
+  l += __shfl_xor(l, 32, 64);
+  if (tok >= T) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  uint16_t* dst = a.out + qoff;
+#pragma unroll
+  for (int c = 0; c < HT; ++c)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint2 w;
+      w.x = pack_bf2(o[c][4 * i] * inv, o[c][4 * i + 1] * inv);
+      w.y = pack_bf2(o[c][4 * i + 2] * inv, o[c][4 * i + 3] * inv);
+      *reinterpret_cast<uint2*>(dst + 32 * c + 8 * i + 4 * h) = w;
+    }
+}
+
+template <int H, int G>
+static int launch_fill(hipStream_t st, const AttnArgs& a) {
+  const int nseq = a.B / a.tpp, tq = 4 * (32 / G);
+  hipLaunchKernelGGL((gqa_fill_kernel<H, G>), dim3(a.Kh, nseq, (a.tpp + tq - 1) / tq), dim3(256), 0, st, a);
+  return check_launch();
+}
+
 template <int H, int G>
 static int launch_attn(hipStream_t st, const AttnArgs& a) {
   hipLaunchKernelGGL((gqa_decode_kernel<H, G>), dim3(a.Kh, a.B, a.nsplit), dim3(AttnWaves<G>::value * 64), 0, st, a);
@@ -225,6 +399,19 @@ int gqa_decode(hipStream_t st, AttnArgs a, int H) {
   if (a.nsplit > 1 && !a.partial) return TMX_ERR_ARG;
   const int G = a.N / a.Kh;
   if (a.N % a.Kh) return TMX_ERR_SHAPE;
+  // several tokens per sequence: one walk over the cache for a block of them (MFMA kernel)
+  if (a.tpp >= kFillMinTokens && a.B % a.tpp == 0 && (size_t)a.C * a.Kh * H * 2 < (1u << 31)) {
+#define TMX_FILL_CASE(HH, GG) \
+  if (H == HH && G == GG) return launch_fill<HH, GG>(st, a);
+    TMX_FILL_CASE(64, 1)
+    TMX_FILL_CASE(64, 2)
+    TMX_FILL_CASE(64, 4)
+    TMX_FILL_CASE(128, 1)
+    TMX_FILL_CASE(128, 2)
+    TMX_FILL_CASE(128, 4)
+    TMX_FILL_CASE(128, 8)
+#undef TMX_FILL_CASE
+  }
 #define TMX_ATTN_CASE(HH, GG) \
   if (H == HH && G == GG) return launch_attn<HH, GG>(st, a);
   TMX_ATTN_CASE(64, 1)
@@ -262,6 +449,26 @@ extern "C" int tmx_gqa_decode_attention(void* stream, const void* q, const void*
   a.out = (uint16_t*)out;
   a.partial = (float*)workspace;
   a.B = B; a.N = N; a.Kh = Kh; a.C = C;
+  a.scale = 1.0f / sqrtf((float)H);
+  return gqa_decode((hipStream_t)stream, a, H);
+}
+
+extern "C" int tmx_gqa_attention_rows(void* stream, const void* q, const void* kcache, const void* vcache,
+                                      const uint8_t* input_mask, const int32_t* step, int buf_len, void* out,
+                                      void* workspace, int n_seq, int T, int N, int Kh, int H, int C) {
+  if (!q || !kcache || !vcache || !input_mask || !step || !out) return TMX_ERR_ARG;
+  if (n_seq <= 0 || T <= 0 || N <= 0 || Kh <= 0 || C <= 0) return TMX_ERR_SHAPE;
+  AttnArgs a = {};
+  a.q = (const uint16_t*)q;
+  a.kcache = (const uint16_t*)kcache;
+  a.vcache = (const uint16_t*)vcache;
+  a.input_mask = input_mask;
+  a.step = step;
+  a.buf_len = buf_len;
+  a.out = (uint16_t*)out;
+  a.partial = (float*)workspace;
+  a.B = n_seq * T; a.N = N; a.Kh = Kh; a.C = C;
+  a.tpp = T;
   a.scale = 1.0f / sqrtf((float)H);
   return gqa_decode((hipStream_t)stream, a, H);
 }
