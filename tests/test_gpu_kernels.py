@@ -49,6 +49,8 @@ def test_int4_dequant_bit_exact_exhaustive():
     # more than 128 rows: 256-row blocks (one partial, several, a ragged tail), with and without K-slices
     (129, 256, 96, 64, 8), (256, 512, 160, 64, 16), (300, 1024, 256, 128, 16), (700, 4096, 512, 64, 32),
     (1024, 2048, 384, 64, 0), (520, 1152, 4096, 128, 16),
+    # unsplit at many rows: LoRA inside the projection's epilogue (ranks 8, 16 and 32, ragged rows)
+    (1024, 256, 12288, 64, 8), (1030, 384, 12288, 128, 32), (1024, 256, 12288, 64, 0),
 ])
 def test_qlora_linear_matches_oracle(M, K, N, group, r):
   T = G.Keep()
@@ -79,6 +81,8 @@ def test_qlora_linear_matches_oracle(M, K, N, group, r):
     # a one-ulp flip of the base or of base + LoRA (before the residual is added) carries through
     # (both at once, in one element of millions: the two add)
     extra = G.ulp_bf16(base) + G.ulp_bf16(out) if (use_res or r) else 0.0
+    if r:  # and a flip of the LoRA delta itself (rank sum in another order), scaled by lora_scale = 2
+      extra = extra + 2.0 * G.ulp_bf16(out - base)
     # sums that cancel to far below their terms: the f32 accumulation error itself (eps32 x sum |x w|)
     extra = extra + 2.0 ** -23 * (np.abs(x) @ np.abs(lin.weight()))
     G.assert_bf16_close(G.host(y), ref, ulps=1.0, extra=extra,

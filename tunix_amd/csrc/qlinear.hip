@@ -1246,6 +1246,49 @@ __device__ __forceinline__ void gemm_block_wide(const QLinearArgs& a, uint16_t* 
   }
   if (!tile_ok) return;
   const int col = nb * 32 + nl;
+  if (!LORA && a.t16) {
+    // LoRA in the epilogue: delta tile [32 rows, 32 columns] = t16 rows . B columns, 16 ranks per
+    // MFMA (t rows are the A operand, so the delta lands in the accumulator layout of acc[m]);
+    // y = bf16(bf16(base) + bf16(bf16(delta) ls))
+    const int seg = nb * 32 >= a.seg_end[0] ? (nb * 32 >= a.seg_end[1] ? 2 : 1) : 0;
+    const int tc0 = seg * a.lora_r;
+    const int nkb = (a.lora_r + 15) >> 4;  // host: <= 4
+    u32x4_t bfr[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      uint32_t w[4] = {0, 0, 0, 0};
+      if (kb < nkb) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int rr = kb * 16 + 8 * h + j;
+          const uint32_t e = rr < a.lora_r ? a.lora_b[(size_t)rr * a.N + col] : 0u;
+          w[j >> 1] |= e << (16 * (j & 1));
+        }
+      }
+      bfr[kb] = u32x4_t{w[0], w[1], w[2], w[3]};
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int trow = row0 + m * 32 + nl;
+      const uint16_t* tp = a.t16 + (size_t)(trow < a.M ? trow : a.M - 1) * a.ldt16 + tc0 + 8 * h;
+      f32x16_t d;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) d[r] = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+        if (kb < nkb) {
+          const bf16x8_t tf = *reinterpret_cast<const bf16x8_t*>(tp + kb * 16);
+          d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf, __builtin_bit_cast(bf16x8_t, bfr[kb]), d, 0, 0, 0);
+        }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = row0 + m * 32 + acc_row(r, lane);
+        if (row >= a.M) continue;
+        a.y_bf16[(size_t)row * a.ldy + col] = f2bf(rbf(acc[m][r]) + rbf(rbf(d[r]) * a.lora_ls));
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -1276,13 +1319,26 @@ __global__ __launch_bounds__(512, 1) void qlinear_mfma_wide_kernel(QLinearArgs a
   else gemm_block_wide<false>(a, smem, bx, by, bz);
 }
 
-static int launch_qlinear_wide(hipStream_t st, QLinearArgs a) {
+// t16[m][c] = bf16(sum of the planes' values) for c < cols, 0 up to the row stride ldt
+__global__ __launch_bounds__(256) void lora_t_reduce_kernel(const float* t_part, int nsplit, int M, int ldt,
+                                                            uint16_t* t16, int cols) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * ldt) return;
+  const int m = i / ldt, c = i - m * ldt;
+  float t = 0.f;
+  if (c < cols)
+    for (int sp = 0; sp < nsplit; ++sp) t += t_part[((size_t)sp * M + m) * ldt + c];
+  t16[(size_t)m * ldt + c] = f2bf(t);
+}
+
+// part: 0 = main blocks and LoRA blocks in one launch, 1 = LoRA blocks only, 2 = main blocks only
+static int launch_qlinear_wide(hipStream_t st, QLinearArgs a, int part = 0) {
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&qlinear_mfma_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
       (int)KW::LDS);
   if (attr != hipSuccess) return TMX_ERR_LAUNCH;
-  a.n_main_blocks = (a.N + KW::COLS - 1) / KW::COLS;
-  const int blocks = a.n_main_blocks + (a.a_t ? a.lora_blocks_per_split : 0);
+  a.n_main_blocks = part == 1 ? 0 : (a.N + KW::COLS - 1) / KW::COLS;
+  const int blocks = a.n_main_blocks + ((a.a_t && part != 2) ? a.lora_blocks_per_split : 0);
   const int row_blocks = (a.M + KW::ROWS - 1) / KW::ROWS;
   int S = 8;
   while (row_blocks % S) S >>= 1;  // gcd(row_blocks, 8)
@@ -1469,6 +1525,51 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   return launch_qlinear<4, 2>(st, a);
 }
 
+int qlinear_wide_lora(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales, const void* a_t,
+                      const void* lora_b, int r, float ls, const int* seg_end, void* y_bf16, float* t_part,
+                      uint16_t* t16, int M, int K, int N, int G, int Rpad) {
+  if (!x || !qw || !scales || !y_bf16) return TMX_ERR_ARG;
+  if (a_t && (!lora_b || !t_part || !t16 || r <= 0)) return TMX_ERR_ARG;
+  if (M <= 128 || K % 128 || N % 32 || G % 64 || (G & (G - 1)) || K % G || ldx % 8) return TMX_ERR_SHAPE;
+  if (a_t && (r % 8 || r > 64 || Rpad <= 0 || Rpad % 32 || Rpad > TMX_MAX_RPAD)) return TMX_ERR_UNSUPPORTED;
+  if (qlinear_num_splits(K, N, M) != 1) return TMX_ERR_UNSUPPORTED;
+  if ((size_t)256 * ldx * 2 >= (1u << 31) || (size_t)K * N / 2 >= (1u << 31) || (size_t)K * Rpad * 2 >= (1u << 31))
+    return TMX_ERR_SHAPE;
+  const int KT = K / 64;
+  QLinearArgs a = {};
+  a.fixed_slice = -1;
+  a.ldy = N;
+  a.x = (const uint16_t*)x;
+  a.ldx = ldx;
+  a.qw = (const uint4*)qw;
+  a.scales = (const uint16_t*)scales;
+  a.a_t = (const uint16_t*)a_t;
+  a.y_bf16 = (uint16_t*)y_bf16;
+  a.t_part = t_part;
+  a.ldt = TMX_MAX_RPAD;
+  a.M = M; a.K = K; a.N = N; a.G = G; a.Rpad = Rpad;
+  a.nsplit = 1;
+  a.kt_per_split = slice_len(KT, 1);
+  const int nls = qlinear_num_lora_splits(K, N);
+  a.lora_blocks_per_split = nls;
+  a.kt_per_lora_split = lora_slice_len(K, N);
+  if (a_t) {
+    if (a.kt_per_lora_split % 2) return TMX_ERR_UNSUPPORTED;
+    int rc = launch_qlinear_wide(st, a, 1);
+    if (rc != TMX_OK) return rc;
+    hipLaunchKernelGGL(lora_t_reduce_kernel, dim3((M * TMX_MAX_RPAD + 255) / 256), dim3(256), 0, st, t_part, nls, M,
+                       TMX_MAX_RPAD, t16, Rpad);
+    if ((rc = check_launch()) != TMX_OK) return rc;
+    a.t16 = t16;
+    a.ldt16 = TMX_MAX_RPAD;
+    a.lora_b = (const uint16_t*)lora_b;
+    a.lora_r = r;
+    a.lora_ls = ls;
+    for (int i = 0; i < 3; ++i) a.seg_end[i] = seg_end ? seg_end[i] : N;
+  }
+  return launch_qlinear_wide(st, a, 2);
+}
+
 // ---------------------------------------------------------------------------
 // Bit-exact dequantisation to a dense bf16 [K, N] matrix (checker / fallback for
 // callers that want the reference's materialised weight).
@@ -1539,7 +1640,9 @@ extern "C" int tmx_int4_dequant(void* stream, const void* qweight, const void* s
 
 extern "C" size_t tmx_qlora_linear_workspace_bytes(int M, int K, int N) {
   const size_t s = qlinear_num_splits(K, N, M);
-  return (s * (size_t)M * N + (size_t)TMX_MAX_LORA_SPLITS * M * TMX_MAX_RPAD) * sizeof(float);
+  // f32 K-slice planes, f32 LoRA planes, bf16 LoRA projection (many rows)
+  return (s * (size_t)M * N + (size_t)TMX_MAX_LORA_SPLITS * M * TMX_MAX_RPAD) * sizeof(float) +
+         (size_t)M * TMX_MAX_RPAD * 2;
 }
 
 extern "C" int tmx_qlora_linear_num_splits(int M, int K, int N) { return qlinear_num_splits(K, N, M); }
@@ -1564,6 +1667,14 @@ extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight
   const int ns = qlinear_num_splits(K, N, M);
   float* y_part = (float*)workspace;
   float* t_part = y_part + (size_t)ns * M * N;
+  if (M > 128 && !residual && ns == 1) {
+    // many rows, unsplit: LoRA in the projection's epilogue
+    uint16_t* t16 = (uint16_t*)(t_part + (size_t)TMX_MAX_LORA_SPLITS * M * TMX_MAX_RPAD);
+    const int seg_end[3] = {N, N, N};
+    const int rc = qlinear_wide_lora(st, x, K, qweight, scales, lora ? lora_a_t : nullptr, lora_b, r, lora_scale,
+                                     seg_end, y, t_part, t16, M, K, N, G, r_pad);
+    if (rc != TMX_ERR_UNSUPPORTED) return rc;
+  }
   int rc = qlinear_base(st, x, K, qweight, scales, lora ? lora_a_t : nullptr, nullptr, y_part, t_part,
                         TMX_MAX_RPAD, M, K, N, G, r_pad, ns);
   if (rc != TMX_OK) return rc;

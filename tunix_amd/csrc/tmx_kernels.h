@@ -27,6 +27,11 @@ struct QLinearArgs {
   const uint16_t* lora_b;  // [lora_r][N] bf16
   int lora_r;
   float lora_ls;
+  // LoRA inside the epilogue of the many-rows kernel: t16 = bf16(x . A) [M][ldt16] computed beforehand;
+  // a column below seg_end[s] (and not below seg_end[s - 1]) uses t columns s lora_r .. s lora_r + lora_r - 1
+  const uint16_t* t16;
+  int ldt16;
+  int seg_end[3];
 };
 
 // Routed experts (Qwen3 MoE): one launch multiplies, for every expert, the rows routed to it.
@@ -197,6 +202,13 @@ int qlinear_num_lora_splits(int K, int N);
 int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
                            int F, int G);
+// Many rows (M > 128), unsplit: y_bf16 = bf16(bf16(x . W) + bf16(bf16(t . B) ls)) in one pass, t = bf16(x . A)
+// computed by a LoRA-only launch of the same kernel and a small reduction (t_part: f32 planes, t16: bf16
+// [M][TMX_MAX_RPAD] scratch).  seg_end: column ends of the fused matrices (q | k | v, gate | up), unused
+// entries = N.  TMX_ERR_UNSUPPORTED when the shape needs K-slices or the rank is not a multiple of 8.
+int qlinear_wide_lora(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales, const void* a_t,
+                      const void* lora_b, int r, float ls, const int* seg_end, void* y_bf16, float* t_part,
+                      uint16_t* t16, int M, int K, int N, int G, int Rpad);
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
                  int N, int G, int Rpad, int nsplit);
