@@ -19,6 +19,7 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 struct Workspace {
   uint16_t *x, *xn, *q, *attn, *act, *y16;
   float *y_part, *t_part, *rope_tab;
+  uint16_t* t16;  // bf16 LoRA projection of a many-rows pass
   float* attn_partial;
   void* head_partial;
   // routed experts (MoE models)
@@ -66,6 +67,7 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   w.y16 = (uint16_t*)take(B * 2 * F * 2);
   w.y_part = (float*)take((size_t)B * ypart * 4);
   w.t_part = (float*)take((size_t)TMX_MAX_LORA_SPLITS * B * TMX_MAX_RPAD * 4);
+  w.t16 = (uint16_t*)take(B > 128 ? (size_t)B * TMX_MAX_RPAD * 2 : 0);
   w.rope_tab = (float*)take((size_t)B * m->head_dim * 4);
   w.attn_partial = (float*)take(attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C));
   w.head_partial = take(head_partial_bytes(B, m->vocab_size));
@@ -170,6 +172,14 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     }
     return li;
   };
+  // Many rows (B > 128): projection + LoRA in one pass into w.y16 where the shape allows it (unsplit,
+  // rank % 8 == 0); returns TMX_ERR_UNSUPPORTED (nothing launched) when the caller must take the planes path.
+  auto wide_linear = [&](const void* x, int ldx, const tmx_qlinear_desc& l, int e0, int e1) {
+    if (B <= 128) return (int)TMX_ERR_UNSUPPORTED;
+    const int seg_end[3] = {e0, e1, l.N};
+    return qlinear_wide_lora(st, x, ldx, l.qweight, l.scales, l.lora_a_t, l.lora_b, l.rank, l.lora_scale, seg_end,
+                             w.y16, w.t_part, w.t16, B, l.K, l.N, l.G, l.r_pad);
+  };
   for (int it = 0; it < n_steps; ++it) {
     {  // embedding gather + first input norm + this step's RoPE table
       RowNormArgs a = {};
@@ -195,14 +205,26 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
                             (!l.gate_up.lora_a_t || (2 * l.gate_up.rank <= 32 && l.gate_up.r_pad == 32));
       uint16_t* kc = (uint16_t*)s->kv_cache + (size_t)(2 * i) * kv_elems;
       uint16_t* vc = kc + kv_elems;
-      TMX_TRY(TMX_K_QKV, qlinear_base(st, w.xn, D, l.qkv.qweight, l.qkv.scales, l.qkv.lora_a_t, nullptr,
-                                      w.y_part, w.t_part, TMX_MAX_RPAD, B, D, QKV, l.qkv.G, l.qkv.r_pad,
-                                      sp.qkv));
+      bool fused;  // this projection ran with LoRA in its epilogue: the consumer reads bf16, no LoRA left
+      {
+        if (prof) prof->before(TMX_K_QKV, st);
+        rc = wide_linear(w.xn, D, l.qkv, NH, NH + Kh * H);
+        fused = rc != TMX_ERR_UNSUPPORTED;
+        if (!fused)
+          rc = qlinear_base(st, w.xn, D, l.qkv.qweight, l.qkv.scales, l.qkv.lora_a_t, nullptr, w.y_part, w.t_part,
+                            TMX_MAX_RPAD, B, D, QKV, l.qkv.G, l.qkv.r_pad, sp.qkv);
+        if (prof) prof->after(TMX_K_QKV, st);
+        if (rc != TMX_OK) return rc;
+      }
       {
         RopeArgs a = {};
-        a.qkv_part = w.y_part;
-        a.nsplit = sp.qkv;
-        a.lora = lora_of(l.qkv, sp.qkv);
+        if (fused) {
+          a.qkv_bf16 = w.y16;
+        } else {
+          a.qkv_part = w.y_part;
+          a.nsplit = sp.qkv;
+          a.lora = lora_of(l.qkv, sp.qkv);
+        }
         a.q_norm_w = (const uint16_t*)l.q_norm_w;
         a.k_norm_w = (const uint16_t*)l.k_norm_w;
         a.positions = s->positions; a.step = s->step; a.buf_len = L; a.tpp = T;
@@ -221,13 +243,25 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         a.scale = 1.0f / sqrtf((float)H);
         TMX_TRY(TMX_K_ATTN, gqa_decode(st, a, H));
       }
-      TMX_TRY(TMX_K_O, qlinear_base(st, w.attn, NH, l.o.qweight, l.o.scales, l.o.lora_a_t, nullptr,
-                                    w.y_part, w.t_part, TMX_MAX_RPAD, B, NH, D, l.o.G, l.o.r_pad, sp.o));
+      {
+        if (prof) prof->before(TMX_K_O, st);
+        rc = wide_linear(w.attn, NH, l.o, D, D);
+        fused = rc != TMX_ERR_UNSUPPORTED;
+        if (!fused)
+          rc = qlinear_base(st, w.attn, NH, l.o.qweight, l.o.scales, l.o.lora_a_t, nullptr, w.y_part, w.t_part,
+                            TMX_MAX_RPAD, B, NH, D, l.o.G, l.o.r_pad, sp.o);
+        if (prof) prof->after(TMX_K_O, st);
+        if (rc != TMX_OK) return rc;
+      }
       {
         RowNormArgs a = {};
-        a.y_part = w.y_part;
-        a.nsplit = sp.o;
-        a.lora = lora_of(l.o, sp.o);
+        if (fused) {
+          a.y_bf16 = w.y16;
+        } else {
+          a.y_part = w.y_part;
+          a.nsplit = sp.o;
+          a.lora = lora_of(l.o, sp.o);
+        }
         a.residual = w.x; a.x_out = w.x;
         a.norm_w = (const uint16_t*)l.norm2_w; a.xn_out = w.xn;
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
@@ -271,28 +305,46 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
               l.gate_up.rank, l.gate_up.lora_scale, w.act, B, D, F, l.gate_up.G));
         } else {
         const bool gu16 = sp.gate_up == 1;
-        TMX_TRY(TMX_K_GATE_UP, qlinear_base(st, w.xn, D, l.gate_up.qweight, l.gate_up.scales,
-                                            l.gate_up.lora_a_t, gu16 ? w.y16 : nullptr, w.y_part, w.t_part,
-                                            TMX_MAX_RPAD, B, D, 2 * F, l.gate_up.G, l.gate_up.r_pad,
-                                            sp.gate_up));
+        {
+          if (prof) prof->before(TMX_K_GATE_UP, st);
+          rc = wide_linear(w.xn, D, l.gate_up, F, 2 * F);
+          fused = rc != TMX_ERR_UNSUPPORTED;
+          if (!fused)
+            rc = qlinear_base(st, w.xn, D, l.gate_up.qweight, l.gate_up.scales, l.gate_up.lora_a_t,
+                              gu16 ? w.y16 : nullptr, w.y_part, w.t_part, TMX_MAX_RPAD, B, D, 2 * F, l.gate_up.G,
+                              l.gate_up.r_pad, sp.gate_up);
+          if (prof) prof->after(TMX_K_GATE_UP, st);
+          if (rc != TMX_OK) return rc;
+        }
         {
           SwigluArgs a = {};
-          a.gu_bf16 = gu16 ? w.y16 : nullptr;
+          a.gu_bf16 = (gu16 || fused) ? w.y16 : nullptr;
           a.gu_part = w.y_part;
           a.nsplit = sp.gate_up;
-          a.lora = lora_of(l.gate_up, sp.gate_up);
+          if (!fused) a.lora = lora_of(l.gate_up, sp.gate_up);
           a.act = w.act; a.F = F;
           TMX_TRY(TMX_K_SWIGLU, swiglu(st, a, B));
         }
         }
-        TMX_TRY(TMX_K_DOWN, qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t,
-                                         nullptr, w.y_part, w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G,
-                                         l.down.r_pad, sp.down));
+        {
+          if (prof) prof->before(TMX_K_DOWN, st);
+          rc = wide_linear(w.act, F, l.down, D, D);
+          fused = rc != TMX_ERR_UNSUPPORTED;
+          if (!fused)
+            rc = qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t, nullptr, w.y_part,
+                              w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G, l.down.r_pad, sp.down);
+          if (prof) prof->after(TMX_K_DOWN, st);
+          if (rc != TMX_OK) return rc;
+        }
         {
           RowNormArgs a = {};
-          a.y_part = w.y_part;
-          a.nsplit = sp.down;
-          a.lora = lora_of(l.down, sp.down);
+          if (fused) {
+            a.y_bf16 = w.y16;
+          } else {
+            a.y_part = w.y_part;
+            a.nsplit = sp.down;
+            a.lora = lora_of(l.down, sp.down);
+          }
           a.residual = w.x; a.x_out = w.x;
           a.norm_w = (const uint16_t*)(i + 1 < m->num_layers ? m->layers[i + 1].norm1_w : m->final_norm_w);
           a.xn_out = w.xn;
