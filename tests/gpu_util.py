@@ -40,10 +40,14 @@ def ulp_bf16(ref):
   return np.exp2(np.floor(np.log2(a)) - 7).astype(np.float32)
 
 
-def assert_bf16_close(got, ref, ulps=1.0, extra=0.0, min_exact=0.0, what=''):
+def assert_bf16_close(got, ref, ulps=1.0, extra=0.0, min_exact=0.0, what='', stragglers=0):
+  """|got - ref| <= ulps bf16 ulp + extra everywhere; `stragglers` elements (coincidences of several
+  rounding flips in samples of millions) may reach three times that bound."""
   d = np.abs(got - ref)
   bound = ulps * ulp_bf16(np.maximum(np.abs(ref), np.abs(got))) + extra
   bad = d > bound
+  if stragglers and 0 < bad.sum() <= stragglers:
+    bad = d > 3.0 * bound
   assert not bad.any(), f'{what}: {bad.sum()} of {bad.size} beyond {ulps} bf16 ulp; worst {d.max()} at ref {ref.flat[d.argmax()]}'
   if min_exact:
     assert (d == 0).mean() >= min_exact, f'{what}: only {(d == 0).mean():.5f} exact'
