@@ -301,7 +301,7 @@ def main():
       symbols.setdefault(sym, []).append(cls_name)
     symbols.update({
         f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention'],
-        f'tmx::head_kernel<{mt}>': ['head_sample'],
+        f'tmx::head_kernel<{min(mt, 2)}>': ['head_sample'],  # 65..128 rows: two launches of the 64-row kernel
     })
     idx = {n: i for i, n in enumerate(CLASS_NAMES)}
     # An event pair around a launch also times the packet processing on both sides of it, so it

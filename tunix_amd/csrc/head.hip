@@ -165,11 +165,11 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
             // repeat the sign and the sort leaves them out.
             const uint32_t zb = __float_as_uint(logit + 0.0f);
             const uint32_t ord = (zb & 0x80000000u) ? ~zb : (zb | 0x80000000u);
-            a.sort_keys[(size_t)row * a.V + v] = ((uint64_t)row << 32) | (uint32_t)~ord;
+            a.sort_keys[(size_t)row * a.V + v] = ((uint64_t)(a.row_off + row) << 32) | (uint32_t)~ord;
             key = z;
           } else {
             uint32_t o0, o1;
-            threefry2x32(key0, key1, 0u, (uint32_t)row * (uint32_t)a.V + (uint32_t)v, o0, o1);
+            threefry2x32(key0, key1, 0u, (uint32_t)(a.row_off + row) * (uint32_t)a.V + (uint32_t)v, o0, o1);
             key = z + gumbel_from_bits(o0 ^ o1);
           }
         }
@@ -431,7 +431,25 @@ int head_logits(hipStream_t st, HeadArgs& a) {
   a.nwg = (a.V + 127) / 128;
   if (a.M <= 32) hipLaunchKernelGGL(head_kernel<1>, dim3(a.nwg), dim3(256), 0, st, a);
   else if (a.M <= 64) hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(head_kernel<4>, dim3(a.nwg), dim3(256), 0, st, a);
+  else {
+    // 65 to 128 rows: two launches of the 64-row kernel (two passes over the head matrix, 2 x 0.27 ms
+    // on a 1 GB head) beat the 128-row instantiation (0.87 ms: one workgroup per CU, its x tile and
+    // weight ring no longer hide the latencies); the partials of both halves sit where one
+    // finalize launch over all rows expects them
+    HeadArgs lo = a, hi = a;
+    lo.M = 64;
+    hi.M = a.M - 64;
+    hi.x = a.x + (size_t)64 * a.D;
+    hi.row_base = a.row_base + 64;
+    hi.row_off = a.row_off + 64;
+    if (a.logits_out) hi.logits_out = a.logits_out + (size_t)64 * a.V;
+    if (a.sort_keys) hi.sort_keys = a.sort_keys + (size_t)64 * a.V;
+    hi.part_f = a.part_f + (size_t)64 * a.nwg * 4;
+    hi.part_i = a.part_i + (size_t)64 * a.nwg;
+    hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, lo);
+    if (hi.M <= 32) hipLaunchKernelGGL(head_kernel<1>, dim3(a.nwg), dim3(256), 0, st, hi);
+    else hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, hi);
+  }
   return check_launch();
 }
 

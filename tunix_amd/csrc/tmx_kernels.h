@@ -159,6 +159,8 @@ struct HeadArgs {
   int buf_len;
   int tpp;  // tokens per pass (0: 1), score mode only: row m is sequence m / tpp at column *step + m % tpp
   int row_base;  // score mode: x holds rows row_base .. row_base + M - 1 of the pass (chunks of <= 128 rows)
+  int row_off;   // set by head_logits when it splits the rows over two launches: x, logits_out, sort_keys and the
+                 // partials point at row row_off of the call, whose index the sort keys and the noise counter use
 };
 
 
