@@ -107,6 +107,8 @@ def main():
   ap.add_argument('--steps', type=int, default=496)
   ap.add_argument('--warmup', type=int, default=16)
   ap.add_argument('--workload', default='llama3.1-8b-grpo', choices=sorted(WORKLOADS))
+  ap.add_argument('--sequences', type=int, default=0,
+                  help='override the number of sequences of the workload (the headline metric is the default)')
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--no-profile', action='store_true')
   ap.add_argument('--graph', action='store_true', help='replay one recorded decode step (tmx_decode_steps_graph)')
@@ -129,6 +131,8 @@ def main():
   sys.path.insert(0, os.path.join(ROOT, 'tests'))
 
   name, batch, prompt, new, group, rank, temp, top_p = WORKLOADS[args.workload]
+  if args.sequences > 0:
+    batch = args.sequences
   if args.steps + args.warmup > new:
     print(f'bench.py: steps + warmup must be <= {new} new tokens of the workload', file=sys.stderr)
     sys.exit(2)

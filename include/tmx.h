@@ -45,7 +45,7 @@ extern "C" {
 #define TMX_MAX_RPAD 128   /* widest padded LoRA projection (sum of fused ranks, rounded up to 32) */
 #define TMX_MAX_SPLITS 16  /* most K-slices a projection is split into */
 #define TMX_MAX_LORA_SPLITS 32 /* most K-slices of the LoRA projection x . A */
-#define TMX_MAX_FILL_ROWS 4096 /* most rows (sequences x tokens) of one cache-fill or scoring pass */
+#define TMX_MAX_FILL_ROWS 4096 /* most rows (sequences x tokens per sequence) of one pass of tmx_decode_steps */
 
 #define TMX_SAMPLE_GREEDY 0
 #define TMX_SAMPLE_TOP_P 1
@@ -273,9 +273,9 @@ typedef struct {
                               sample == 0, or TMX_SAMPLE_SCORE): every pass consumes the T tokens at
                               columns *step .. *step + T - 1 of each sequence as batch * T rows, each
                               attending to the slots up to its own column; *step advances by T.
-                              Rows: <= 128 for MoE models; a cache fill or scoring pass of a dense
-                              model takes up to TMX_MAX_FILL_ROWS when every projection has
-                              K % 128 == 0 (the head scores them in chunks of 128).
+                              Rows of a pass (batch * T, also for T <= 1): <= 128 for MoE models; a
+                              dense model takes up to TMX_MAX_FILL_ROWS when every projection has
+                              K % 128 == 0.
                               The workspace must be sized for batch * T rows. */
 } tmx_decode_state;
 

@@ -152,6 +152,52 @@ def test_temperature_sampling_follows_the_threefry_schedule():
   assert all((a == b).all() for a, b in zip(out.tokens, out3.tokens))
 
 
+def test_batches_over_128_sequences():
+  """More than 128 sequences per step: the projections run in 256-row blocks, the head takes the
+  rows 64 at a time.  Greedy rows spread over the batch against the oracle (a sequence does not
+  depend on its neighbours), temperature sampling against the threefry schedule over all rows
+  (the noise counter is row * V + v), top-p through the sorting branch."""
+  cfg = C.TOY
+  oracle, model = _pair(cfg, seed=11, targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
+  rng = np.random.default_rng(6)
+  nb = 150
+  prompts = [rng.integers(3, cfg.vocab_size, 3 + (i * 7) % 10) for i in range(nb)]
+  s = _sampler(model, cfg, 32)
+  out = s(prompt_token_ids=prompts, max_generation_steps=8, return_logprobs=True, eos_tokens=[-1])
+  assert len(out.tokens) == nb
+  rows = [0, 31, 63, 64, 100, 127, 128, 129, 149]
+  ref = OSAM.generate(oracle, cfg, [prompts[i] for i in rows], 8, 32, eos_ids=(-1,))
+  class _Sub:
+    tokens = [out.tokens[i] for i in rows]
+    logprobs = [out.logprobs[i] for i in rows]
+  _compare_greedy(_Sub, ref, len(rows), 40)
+  # temperature sampling: every row follows categorical(fold_in(key, step), logits / T) on its own logits
+  prompts8 = [rng.integers(3, cfg.vocab_size, 8) for _ in range(nb)]  # equal lengths: one decoding step index
+  out = s(prompt_token_ids=prompts8, max_generation_steps=4, return_logprobs=True, return_logits=True,
+          eos_tokens=[-1], temperature=0.9, top_p=1.0, seed=7)
+  key0 = prng.prng_key(7)
+  agree = total = 0
+  for step in range(4):
+    z = np.stack([out.logits[b][step] for b in range(nb)]).astype(np.float32) / np.float32(0.9)
+    noisy = z + prng.gumbel(prng.fold_in(key0, 8 - 1 + step), z.shape)
+    srt = np.sort(noisy, axis=-1)
+    clear = (srt[:, -1] - srt[:, -2]) > 1e-4
+    got = np.array([out.tokens[b][step] for b in range(nb)])
+    np.testing.assert_array_equal(got[clear], np.argmax(noisy, -1)[clear])
+    agree += clear.sum()
+    total += nb
+    want_lp = OS.log_softmax(z)[np.arange(nb), got]
+    np.testing.assert_allclose([out.logprobs[b][step] for b in range(nb)], want_lp, atol=3e-5)
+  assert agree >= total - 8
+  # the sorting branch (top-p < 1): tokens come from the nucleus of the row's own logits
+  out = s(prompt_token_ids=prompts8, max_generation_steps=3, return_logits=True, eos_tokens=[-1],
+          temperature=1.0, top_p=0.5, seed=3)
+  for b in (0, 64, 128, 149):
+    for step in range(3):
+      members = OS.nucleus_members(np.asarray(out.logits[b][step], np.float32), 0.5)
+      assert out.tokens[b][step] in members, (b, step)
+
+
 def test_top_p_and_top_k_sampling_follow_the_reference_rule():
   """The sorting branch of sample_top_p (tunix/generate/sampler.py:136-153) through the whole
   Sampler: every token equals the oracle's draw on the kernel's own logits of that step."""

@@ -119,14 +119,13 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   // rows of a pass: one per sequence, or tokens_per_pass consecutive tokens of every sequence
   // (cache fill and scoring only: sampling needs the previous token)
   const int NSEQ = s->batch, T = s->tokens_per_pass > 1 ? s->tokens_per_pass : 1;
-  if (NSEQ <= 0 || NSEQ > 128 || T > 128) return TMX_ERR_SHAPE;
+  if (NSEQ <= 0 || NSEQ > TMX_MAX_FILL_ROWS || T > 128) return TMX_ERR_SHAPE;
   if (T > 1 && sample && s->sampling_mode != TMX_SAMPLE_SCORE) return TMX_ERR_ARG;
   const int B = NSEQ * T, C = s->cache_size, L = s->buf_len;
-  // choosing tokens takes up to 128 rows; a cache-fill or scoring pass of a dense model up to
-  // TMX_MAX_FILL_ROWS, which the projections multiply in 256-row blocks (every K % 128 == 0) and
-  // the head scores in chunks of 128 rows
-  const bool choose = sample && s->sampling_mode != TMX_SAMPLE_SCORE;
-  if (B > ((choose || moe) ? 128 : TMX_MAX_FILL_ROWS) || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
+  // a pass takes up to TMX_MAX_FILL_ROWS rows; above 128 rows the projections multiply in 256-row
+  // blocks (dense models, every K % 128 == 0), the head takes its rows 64 at a time (scoring: 256 x 256
+  // blocks); MoE models stay at 128 rows
+  if (B > (moe ? 128 : TMX_MAX_FILL_ROWS) || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
   if (moe && (m->experts_per_tok <= 0 || m->experts_per_tok > m->num_experts ||
               (size_t)B * m->experts_per_tok > 1024))
     return TMX_ERR_SHAPE;
@@ -354,7 +353,8 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       }
       if (prof) TMX_TRY(TMX_K_EMPTY, empty_launch(st));
     }
-    if (sample && B > 128 && !s->logits_out && s->n_forbidden == 0 && D % 128 == 0) {
+    if (sample && s->sampling_mode == TMX_SAMPLE_SCORE && B > 128 && !s->logits_out && s->n_forbidden == 0 &&
+        D % 128 == 0) {
       // a scoring pass of many rows: the matrix-pipe-bound head kernel
       HeadArgs a = {};
       a.x = w.xn;
@@ -372,33 +372,30 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       a.tpp = T;
       TMX_TRY(TMX_K_HEAD, head_score_wide(st, a));
     } else if (sample) {
-      for (int r0 = 0; r0 < B; r0 += 128) {  // one chunk unless a scoring pass has more than 128 rows
-        HeadArgs a = {};
-        a.x = w.xn + (size_t)r0 * D;
-        a.row_base = r0;
-        a.w = (const uint16_t*)m->head;
-        a.M = B - r0 < 128 ? B - r0 : 128; a.D = D; a.V = m->vocab_size;
-        a.mode = s->sampling_mode;
-        a.temperature = s->temperature;
-        a.k0 = s->seed_hi; a.k1 = s->seed_lo;
-        a.step = s->step;
-        a.forbidden = s->forbidden; a.n_forbidden = s->n_forbidden;
-        a.logits_out = s->logits_out ? s->logits_out + (size_t)r0 * m->vocab_size : nullptr;
-        const size_t nwg = (m->vocab_size + 127) / 128;
-        a.part_f = (float*)w.head_partial;
-        a.part_i = (int32_t*)((float*)w.head_partial + (size_t)a.M * nwg * 4);
-        a.token_buffer = s->token_buffer;
-        a.logprobs = s->logprobs;
-        a.done = s->done;
-        a.eos = s->eos_ids; a.n_eos = s->n_eos;
-        a.buf_len = L;
-        a.tpp = T;
-        if (nucleus) {
-          TMX_TRY(TMX_K_HEAD, head_sample_nucleus(st, a, s->top_p, s->top_k, s->nucleus_workspace,
-                                                  s->nucleus_workspace_bytes));
-        } else {
-          TMX_TRY(TMX_K_HEAD, head_sample(st, a));
-        }
+      HeadArgs a = {};
+      a.x = w.xn;
+      a.w = (const uint16_t*)m->head;
+      a.M = B; a.D = D; a.V = m->vocab_size;
+      a.mode = s->sampling_mode;
+      a.temperature = s->temperature;
+      a.k0 = s->seed_hi; a.k1 = s->seed_lo;
+      a.step = s->step;
+      a.forbidden = s->forbidden; a.n_forbidden = s->n_forbidden;
+      a.logits_out = s->logits_out;
+      const size_t nwg = (m->vocab_size + 127) / 128;
+      a.part_f = (float*)w.head_partial;
+      a.part_i = (int32_t*)((float*)w.head_partial + (size_t)B * nwg * 4);
+      a.token_buffer = s->token_buffer;
+      a.logprobs = s->logprobs;
+      a.done = s->done;
+      a.eos = s->eos_ids; a.n_eos = s->n_eos;
+      a.buf_len = L;
+      a.tpp = T;
+      if (nucleus) {
+        TMX_TRY(TMX_K_HEAD, head_sample_nucleus(st, a, s->top_p, s->top_k, s->nucleus_workspace,
+                                                s->nucleus_workspace_bytes));
+      } else {
+        TMX_TRY(TMX_K_HEAD, head_sample(st, a));
       }
     }
     TMX_TRY(TMX_K_ADVANCE, advance_step(st, s->step, T));

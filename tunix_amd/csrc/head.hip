@@ -427,28 +427,24 @@ int head_score_wide(hipStream_t st, HeadArgs a) {
 }
 
 int head_logits(hipStream_t st, HeadArgs& a) {
-  if (a.V % 32 || a.D % 64 || a.M <= 0 || a.M > 128) return TMX_ERR_SHAPE;
+  if (a.V % 32 || a.D % 64 || a.M <= 0 || a.M > TMX_MAX_FILL_ROWS) return TMX_ERR_SHAPE;
   a.nwg = (a.V + 127) / 128;
-  if (a.M <= 32) hipLaunchKernelGGL(head_kernel<1>, dim3(a.nwg), dim3(256), 0, st, a);
-  else if (a.M <= 64) hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, a);
-  else {
-    // 65 to 128 rows: two launches of the 64-row kernel (two passes over the head matrix, 2 x 0.27 ms
-    // on a 1 GB head) beat the 128-row instantiation (0.87 ms: one workgroup per CU, its x tile and
-    // weight ring no longer hide the latencies); the partials of both halves sit where one
-    // finalize launch over all rows expects them
-    HeadArgs lo = a, hi = a;
-    lo.M = 64;
-    hi.M = a.M - 64;
-    hi.x = a.x + (size_t)64 * a.D;
-    hi.row_base = a.row_base + 64;
-    hi.row_off = a.row_off + 64;
-    if (a.logits_out) hi.logits_out = a.logits_out + (size_t)64 * a.V;
-    if (a.sort_keys) hi.sort_keys = a.sort_keys + (size_t)64 * a.V;
-    hi.part_f = a.part_f + (size_t)64 * a.nwg * 4;
-    hi.part_i = a.part_i + (size_t)64 * a.nwg;
-    hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, lo);
-    if (hi.M <= 32) hipLaunchKernelGGL(head_kernel<1>, dim3(a.nwg), dim3(256), 0, st, hi);
-    else hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, hi);
+  // Rows go through the 32- or 64-row kernel in chunks of 64: one pass over the head matrix per chunk.
+  // (A 128-row instantiation ran 0.87 ms on a 1 GB head against 2 x 0.27 ms: one workgroup per CU, its
+  // x tile and weight ring no longer hide the latencies.)  The partials of every chunk sit where one
+  // finalize launch over all rows expects them.
+  for (int r0 = 0; r0 < a.M; r0 += 64) {
+    HeadArgs c = a;
+    c.M = a.M - r0 < 64 ? a.M - r0 : 64;
+    c.x = a.x + (size_t)r0 * a.D;
+    c.row_base = a.row_base + r0;
+    c.row_off = a.row_off + r0;
+    if (a.logits_out) c.logits_out = a.logits_out + (size_t)r0 * a.V;
+    if (a.sort_keys) c.sort_keys = a.sort_keys + (size_t)r0 * a.V;
+    c.part_f = a.part_f + (size_t)r0 * a.nwg * 4;
+    c.part_i = a.part_i + (size_t)r0 * a.nwg;
+    if (c.M <= 32) hipLaunchKernelGGL(head_kernel<1>, dim3(a.nwg), dim3(256), 0, st, c);
+    else hipLaunchKernelGGL(head_kernel<2>, dim3(a.nwg), dim3(256), 0, st, c);
   }
   return check_launch();
 }

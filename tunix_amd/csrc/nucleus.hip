@@ -180,7 +180,7 @@ size_t nucleus_bytes(int M, int V) {
 }
 
 int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void* ws, size_t ws_bytes) {
-  if (a.V % 32 || a.D % 64 || a.M <= 0 || a.M > 128) return TMX_ERR_SHAPE;
+  if (a.V % 32 || a.D % 64 || a.M <= 0 || a.M > TMX_MAX_FILL_ROWS) return TMX_ERR_SHAPE;
   if (!ws || !(top_p >= 0.f)) return TMX_ERR_ARG;
   size_t sort_tmp = 0;
   if (sort_rows(nullptr, sort_tmp, nullptr, nullptr, nullptr, a.M, a.V, st) != hipSuccess)
