@@ -281,8 +281,8 @@ def main():
     dense = [('qkv_linear', 'qkv'), ('o_linear', 'o')]
     symbols = {}
     if cfg.num_experts:
-      symbols['tmx::moe_expert_kernel<false>'] = ['gate_up_linear']
-      symbols['tmx::moe_expert_kernel<true>'] = ['down_linear']
+      symbols['tmx::moe_stream_kernel<false>'] = ['gate_up_linear']
+      symbols['tmx::moe_stream_kernel<true>'] = ['down_linear']
     else:
       gu = layer0['gate_up']
       fused = (tot_cnt[CLASS_NAMES.index('swiglu')] == 0 and gu.k % 256 == 0 and gu.k < 8192)

@@ -5,7 +5,7 @@
 //   weights, experts = lax.top_k(p, k)        (ties: lower expert id first)
 //   weights = bf16(weights / sum(weights))
 // One workgroup per token.  The expert matrices themselves are multiplied by
-// moe_expert_kernel (qlinear.hip); the weighted sum over a token's experts is taken by the
+// moe_stream_kernel (qlinear.hip); the weighted sum over a token's experts is taken by the
 // row kernel that also adds the residual and normalises (glue.hip).
 #include "tmx_kernels.h"
 

@@ -340,20 +340,28 @@ static int launch_qlinear4(hipStream_t st, QLinearArgs a) {
   return check_launch();
 }
 
-// Routed experts: grid (column blocks, experts).  Every workgroup first collects the pairs
-// (token, slot) routed to its expert from the routing table (at most a few hundred entries),
-// leaves if there are none (so unrouted experts are never streamed), and otherwise runs the
-// 4-wave block over its rows in chunks of 32 with gathered activation rows and scattered
-// output rows.  DOWN = false fuses SwiGLU: the workgroup owns 64 gate columns and the matching
-// 64 up columns.  tunix/models/qwen3/model.py:894-939 evaluated for routed pairs only.
+// Routed experts (tunix/models/qwen3/model.py:894-939 evaluated for routed pairs only): grid (column
+// groups, experts).  Every workgroup first collects the pairs (token, slot) routed to its expert from
+// the routing table (at most a few hundred entries) and leaves if there are none, so unrouted experts
+// are never streamed.  In decode an expert sees a handful of rows (batch x top_k pairs spread over many
+// experts), so the product is nothing but a weight stream: every wave walks its own column tiles (DOWN)
+// or gate / up tile pairs (SwiGLU in its epilogue) over all of K with no LDS and no barrier after the
+// compaction.  Weight tiles come through a ring of kMoeRing tiles per wave (buffer loads, scalar
+// offsets), the x fragments of the live rows straight from global memory (gathered activation rows;
+// lanes of absent rows hold zeros), one k-tile ahead; output rows are scattered.  The ring runs on
+// across the wave's tiles, so the stream never drains.  More than 32 rows of an expert are taken in
+// chunks of 32, each streaming the weights again (rare).
+constexpr int kMoeRing = 4;  // divides K / 64 (K % 256 == 0), so a ring slot is k-tile % 4 in every unit
+
 template <bool DOWN>
-__global__ __launch_bounds__(256, 2) void moe_expert_kernel(MoeArgs m) {
-  __shared__ __align__(16) uint16_t xs[2][32][kXStride];
+__global__ __launch_bounds__(256, 2) void moe_stream_kernel(MoeArgs m) {
   __shared__ int rows_s[1024];
-  __shared__ int src_s[32], dst_s[32];
   __shared__ int wave_cnt[4];
   __shared__ int n_s;
-  const int e = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int TPU = DOWN ? 1 : 2;  // tiles per unit: one column tile, or a gate tile and its up tile
+  const int e = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, nl = lane & 31;
   int base = 0;
   for (int p0 = 0; p0 < m.P; p0 += 256) {  // ordered compaction of { p : expert_of[p] == e }
     const int p = p0 + tid;
@@ -371,31 +379,90 @@ __global__ __launch_bounds__(256, 2) void moe_expert_kernel(MoeArgs m) {
   __syncthreads();
   const int n = n_s;
   if (n == 0) return;
-  QLinearArgs a = {};
-  a.x = m.x;
-  a.ldx = m.ldx;
-  a.qw = m.qw + (size_t)e * m.qw_stride;
-  a.scales = m.scales + (size_t)e * m.sc_stride;
-  a.y_bf16 = m.out;
-  a.ldy = m.ldo;
-  a.K = m.K; a.N = m.N; a.G = m.G;
-  a.n_main_blocks = gridDim.x;
-  a.nsplit = 1;
-  a.kt_per_split = m.K >> 6;
-  a.fixed_slice = 0;
-  a.row_src = src_s;
-  a.row_dst = dst_s;
-  a.pair_off = DOWN ? 0 : (m.N >> 6);  // tiles in F = N / 2 columns
+
+  const int KT = m.K >> 6, KG = m.K / m.G, gs = __builtin_ctz(m.G >> 6);
+  const int NT = m.N >> 5;
+  const int units = DOWN ? NT : NT / 2;  // column tiles, or gate | up pairs (F / 32)
+  // units of this wave: u = blockIdx.x + groups * (wave + 4 j), j = 0, 1, ... (groups = gridDim.x)
+  const int u0 = (int)blockIdx.x + (int)gridDim.x * wave, ustride = (int)gridDim.x * 4;
+  if (u0 >= units) return;
+  const int nu = (units - u0 + ustride - 1) / ustride;
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(m.qw + (size_t)e * m.qw_stride, (uint32_t)NT * KT * 1024u);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.scales + (size_t)e * m.sc_stride, (uint32_t)NT * KG * 64u);
+
   for (int c0 = 0; c0 < n; c0 += 32) {
-    if (tid < 32 && c0 + tid < n) {
-      const int p = rows_s[c0 + tid];
-      src_s[tid] = DOWN ? p : p / m.top_k;
-      dst_s[tid] = p;
+    const int rows = n - c0 < 32 ? n - c0 : 32;
+    // A fragments: lane (row nl, h) reads x[src][64 kt + 16 t + 8 h ..]; absent rows stay zero
+    const bool live = nl < rows;
+    const int pr = live ? rows_s[c0 + nl] : 0;
+    const uint16_t* xrow = m.x + (size_t)(DOWN ? pr : pr / m.top_k) * m.ldx + 8 * h;
+    u32x4_t wring[kMoeRing][TPU];
+    uint16_t sring[kMoeRing][TPU];
+    // tile (unit ui of this wave, k-tile kt) into ring slot sl; past the last unit: its last tile again
+    auto load_w = [&](int ui, int kt, auto sc) __attribute__((always_inline)) {
+      constexpr int sl = decltype(sc)::value;
+      if (ui >= nu) { ui = nu - 1; kt = KT - 1; }
+#pragma unroll
+      for (int c = 0; c < TPU; ++c) {
+        const int nb = u0 + ui * ustride + c * units;  // the gate tile, or the up tile F / 32 further on
+        wring[sl][c] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16, (nb * KT + kt) * 1024, 0);
+        sring[sl][c] = __builtin_amdgcn_raw_buffer_load_b16(rs, nl * 2, (nb * KG + (kt >> gs)) * 64, 0);
+      }
+    };
+    u32x4_t xq[2][4];
+    auto load_x = [&](int kt, int slot) __attribute__((always_inline)) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        xq[slot][t] = live ? *reinterpret_cast<const u32x4_t*>(xrow + kt * 64 + 16 * t) : u32x4_t{0, 0, 0, 0};
+    };
+    static_for<kMoeRing>([&](auto sc) __attribute__((always_inline)) { load_w(0, decltype(sc)::value, sc); });
+    load_x(0, 0);
+    f32x16_t acc[TPU];
+    for (int u = 0; u < nu; ++u) {
+#pragma unroll
+      for (int c = 0; c < TPU; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[c][r] = 0.f;
+      for (int k0 = 0; k0 < KT; k0 += kMoeRing) {  // host: K % 256 == 0, so every group is whole
+        static_for<kMoeRing>([&](auto sc) __attribute__((always_inline)) {
+          constexpr int sl = decltype(sc)::value;
+          const int kt = k0 + sl;
+          load_x(kt + 1 < KT ? kt + 1 : 0, (sl & 1) ^ 1);  // the next k-tile (of the next unit: the same rows)
+          u32x4_t wc[TPU];
+          float s_c[TPU];
+#pragma unroll
+          for (int c = 0; c < TPU; ++c) { wc[c] = wring[sl][c]; s_c[c] = bf2f(sring[sl][c]); }
+          // slot consumed: refill it with the tile kMoeRing steps on in the wave's unit-major order
+          if (kt + kMoeRing < KT) load_w(u, kt + kMoeRing, sc);
+          else load_w(u + 1, kt + kMoeRing - KT, sc);
+#pragma unroll
+          for (int c = 0; c < TPU; ++c) {
+            const float m8s = -8.f * s_c[c];
+            const uint32_t wd[4] = {wc[c].x, wc[c].y, wc[c].z, wc[c].w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, xq[sl & 1][t]),
+                                                               dequant_word(wd[t], s_c[c], m8s), acc[c], 0, 0, 0);
+          }
+        });
+      }
+      // epilogue of the unit
+      const int ut = u0 + u * ustride;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = acc_row(r, lane);
+        if (row >= rows) continue;
+        const int p = rows_s[c0 + row];
+        if (DOWN) {
+          m.out[(size_t)p * m.ldo + ut * 32 + nl] = f2bf(acc[0][r]);
+        } else {
+          const float g = rbf(acc[0][r]), up = rbf(acc[TPU - 1][r]);
+          const float sg = rbf(1.f / (1.f + expf(-g)));
+          m.out[(size_t)p * m.ldo + ut * 32 + nl] = f2bf(rbf(g * sg) * up);
+        }
+      }
     }
-    __syncthreads();
-    a.M = n - c0 < 32 ? n - c0 : 32;
-    gemm_block4<1, false>(a, xs);
-    __syncthreads();
   }
 }
 
@@ -403,13 +470,16 @@ int moe_experts(hipStream_t st, const MoeArgs& a, int E, bool down) {
   if (!a.x || !a.qw || !a.scales || !a.expert_of || !a.out) return TMX_ERR_ARG;
   if (a.P <= 0 || a.P > 1024 || a.top_k <= 0 || E <= 0) return TMX_ERR_SHAPE;
   if (a.K % 256 || a.G % 64 || (a.G & (a.G - 1)) || a.K % a.G || a.ldx % 8) return TMX_ERR_SHAPE;
-  if (down) {
-    if (a.N % 128) return TMX_ERR_SHAPE;
-    hipLaunchKernelGGL(moe_expert_kernel<true>, dim3(a.N / 128, E), dim3(256), 0, st, a);
-  } else {
-    if (a.N % 128) return TMX_ERR_SHAPE;  // F % 64 == 0
-    hipLaunchKernelGGL(moe_expert_kernel<false>, dim3(a.N / 128, E), dim3(256), 0, st, a);
-  }
+  if (a.N % 128) return TMX_ERR_SHAPE;  // gate | up: F % 64 == 0
+  // decode: few rows per expert, a pure weight stream
+  // column groups per expert: one gate | up pair (2 x K / 64 weight tiles) or two down tiles per wave
+  // (measured on the 30B-A3B shapes: 6 groups for gate | up, 8 for down; fewer leave CUs short of
+  // loads in flight, more leave waves without work)
+  const int units = down ? a.N / 32 : a.N / 64;
+  int groups = units / (down ? 8 : 4);
+  groups = groups < 1 ? 1 : (groups > 32 ? 32 : groups);
+  if (down) hipLaunchKernelGGL(moe_stream_kernel<true>, dim3(groups, E), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(moe_stream_kernel<false>, dim3(groups, E), dim3(256), 0, st, a);
   return check_launch();
 }
 
