@@ -353,24 +353,25 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       }
       if (prof) TMX_TRY(TMX_K_EMPTY, empty_launch(st));
     }
-    if (sample && s->sampling_mode == TMX_SAMPLE_SCORE && B > 128 && !s->logits_out && s->n_forbidden == 0 &&
-        D % 128 == 0) {
-      // a scoring pass of many rows: the matrix-pipe-bound head kernel
+    if (sample && !nucleus && B > 128 && !s->logits_out && s->n_forbidden == 0 && D % 128 == 0) {
+      // many rows: the matrix-pipe-bound head kernel
       HeadArgs a = {};
       a.x = w.xn;
       a.w = (const uint16_t*)m->head;
       a.M = B; a.D = D; a.V = m->vocab_size;
       a.mode = s->sampling_mode;
       a.temperature = s->temperature;
+      a.k0 = s->seed_hi; a.k1 = s->seed_lo;
       a.step = s->step;
       a.part_f = (float*)w.head_partial;
       a.part_i = (int32_t*)((float*)w.head_partial + (size_t)B * ((m->vocab_size + 255) / 256) * 4);
       a.token_buffer = s->token_buffer;
       a.logprobs = s->logprobs;
       a.done = s->done;
+      a.eos = s->eos_ids; a.n_eos = s->n_eos;
       a.buf_len = L;
       a.tpp = T;
-      TMX_TRY(TMX_K_HEAD, head_score_wide(st, a));
+      TMX_TRY(TMX_K_HEAD, head_wide(st, a));
     } else if (sample) {
       HeadArgs a = {};
       a.x = w.xn;

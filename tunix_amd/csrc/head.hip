@@ -268,8 +268,8 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Scoring passes with many rows (teacher forcing over whole sequences): the same product as a
-// matrix-pipe-bound kernel.  A workgroup multiplies 256 vocabulary rows by 256 sequence rows:
+// Many rows (scoring passes over whole sequences, decode steps of more than 128 sequences): the same
+// product as a matrix-pipe-bound kernel.  A workgroup multiplies 256 vocabulary rows by 256 sequence rows:
 // the vocabulary rows are the A operand and come through a double-buffered LDS slab filled by
 // direct-to-LDS loads (256-byte rows of a 128-wide k-step, chunks XOR-swizzled by row % 16);
 // wave w owns sequence rows 32 w .. 32 w + 31 as the B operand, read straight from global
@@ -284,7 +284,7 @@ struct HW {
   static constexpr size_t LDS = (size_t)2 * ROWS * XS * 2;  // 128 KiB
 };
 
-__global__ __launch_bounds__(512, 1) void head_score_wide_kernel(HeadArgs a, int tok_blocks, int voc_blocks) {
+__global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_blocks, int voc_blocks) {
   extern __shared__ __align__(16) uint16_t smem[];
   constexpr int MT = HW::MT, TS = HW::TS, XS = HW::XS, ROWS = HW::ROWS;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -373,27 +373,42 @@ __global__ __launch_bounds__(512, 1) void head_score_wide_kernel(HeadArgs a, int
     wait_slab();
   }
 
-  // per sequence row: running max and sum of exp over this block's vocabulary rows, and the z of
-  // the given next token if it lies in the block (key 0 marks it, as in head_kernel's score mode)
+  // per sequence row: running max and sum of exp over this block's vocabulary rows and the best
+  // candidate by key, as in head_kernel: greedy key = logit; sampling key = z + Gumbel noise of the
+  // counter row * V + v; scoring: the given next token (key 0 marks it)
+  const bool score = a.mode == TMX_SAMPLE_SCORE, sampling = a.mode == TMX_SAMPLE_TOP_P;
+  uint32_t key0 = 0, key1 = 0;
+  if (sampling) threefry2x32(a.k0, a.k1, 0u, (uint32_t)*a.step, key0, key1);
   const int tpp = a.tpp > 0 ? a.tpp : 1;
-  const int target = a.token_buffer[(size_t)(tok_l / tpp) * a.buf_len + *a.step + tok_l % tpp + 1];
+  const int target = score ? a.token_buffer[(size_t)(tok_l / tpp) * a.buf_len + *a.step + tok_l % tpp + 1] : -1;
   float mx = kNegBig, se = 0.f;
   Best best = {-INFINITY, -INFINITY, 0x7FFFFFFF};
-#pragma unroll
-  for (int m = 0; m < MT; ++m)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
+  // (unrolled by construction: a loop the compiler declines to unroll would index the accumulators
+  // dynamically and move them to scratch memory)
+  static_for<MT * 16>([&](auto ic) __attribute__((always_inline)) {
+      constexpr int m = decltype(ic)::value / 16, r = decltype(ic)::value % 16;
       const int v = v0 + m * 32 + acc_row(r, lane);
-      if (v >= a.V) continue;
-      const float z = rbf(acc[m][r]) / a.temperature;
+      if (v >= a.V) return;
+      const float logit = rbf(acc[m][r]);
+      float z = logit, key = logit;
+      if (score) {
+        z = logit / a.temperature;
+        key = (v == target) ? 0.f : -INFINITY;
+      } else if (sampling) {
+        z = logit / a.temperature;
+        uint32_t o0, o1;
+        threefry2x32(key0, key1, 0u, (uint32_t)tok_l * (uint32_t)a.V + (uint32_t)v, o0, o1);
+        key = z + gumbel_from_bits(o0 ^ o1);
+      }
       if (z > mx) {
         se = se * expf(mx - z) + 1.f;
         mx = z;
       } else {
         se += expf(z - mx);
       }
-      if (v == target) best = {0.f, z, v};
-    }
+      Best c = {key, z, v};
+      best_merge(best, c);
+  });
   {
     const float mx2 = __shfl_xor(mx, 32, 64), se2 = __shfl_xor(se, 32, 64);
     Best o = {__shfl_xor(best.key, 32, 64), __shfl_xor(best.z, 32, 64), __shfl_xor(best.idx, 32, 64)};
@@ -407,18 +422,18 @@ __global__ __launch_bounds__(512, 1) void head_score_wide_kernel(HeadArgs a, int
   }
 }
 
-// Scoring of M rows (any count) with the wide kernel + the finalize kernel; the caller has checked
-// mode == TMX_SAMPLE_SCORE, no forbidden ids, no logits output, D % 128 == 0.
-int head_score_wide(hipStream_t st, HeadArgs a) {
+// M rows (any count) with the wide kernel + the finalize kernel: greedy, sampling without the sorting
+// branch, or scoring; the caller has checked: no forbidden ids, no logits output, D % 128 == 0.
+int head_wide(hipStream_t st, HeadArgs a) {
   if (a.D % 128 || a.M <= 0 || (size_t)a.M * a.D * 2 >= (1u << 31) || (size_t)256 * a.D * 2 >= (1u << 31))
     return TMX_ERR_SHAPE;
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&head_score_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)HW::LDS);
+      reinterpret_cast<const void*>(&head_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)HW::LDS);
   if (attr != hipSuccess) return TMX_ERR_LAUNCH;
   const int tok_blocks = (a.M + 255) / 256, voc_blocks = (a.V + HW::ROWS - 1) / HW::ROWS;
   a.nwg = voc_blocks;
   a.row_base = 0;
-  hipLaunchKernelGGL(head_score_wide_kernel, dim3(tok_blocks * voc_blocks), dim3(512), HW::LDS, st, a, tok_blocks,
+  hipLaunchKernelGGL(head_wide_kernel, dim3(tok_blocks * voc_blocks), dim3(512), HW::LDS, st, a, tok_blocks,
                      voc_blocks);
   int rc = check_launch();
   if (rc != TMX_OK) return rc;

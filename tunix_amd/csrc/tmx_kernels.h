@@ -192,9 +192,9 @@ size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
 int moe_route(hipStream_t st, const RouterArgs& a, int B);
 int moe_experts(hipStream_t st, const MoeArgs& a, int E, bool down);
 int head_sample(hipStream_t st, HeadArgs a);
-// score mode over any number of rows (256 x 256 blocks); needs D % 128 == 0, no forbidden ids, no logits output;
-// part_f / part_i sized [M][ceil(V / 256)]
-int head_score_wide(hipStream_t st, HeadArgs a);
+// any number of rows in 256 x 256 blocks (greedy, sampling without the sorting branch, scoring); needs
+// D % 128 == 0, no forbidden ids, no logits output; part_f / part_i sized [M][ceil(V / 256)]
+int head_wide(hipStream_t st, HeadArgs a);
 int head_logits(hipStream_t st, HeadArgs& a);  // the vocabulary kernel alone; fills a.nwg
 int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void* ws, size_t ws_bytes);
 size_t nucleus_bytes(int M, int V);
