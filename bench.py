@@ -300,12 +300,18 @@ def main():
       if pl.k % 256 == 0:
         return f'tmx::qlinear_mfma_dma_kernel<{mt}>'
       return f'tmx::qlinear_mfma_kernel<{mt}, 2>'
+    if batch > 128 and not cfg.num_experts:
+      # more than 128 sequences (--sequences): every projection runs the 256-row kernel, the head in
+      # 256 x 256 blocks (the byte-based fractions below then understate these MFMA-bound kernels)
+      symbols = {'tmx::qlinear_mfma_wide_kernel': ['qkv_linear', 'o_linear', 'gate_up_linear', 'down_linear']}
+      dense = []
     for cls_name, key in dense:
       sym = f'tmx::qlinear_mfma4_kernel<{mt}>' if four(layer0[key]) else kway_symbol(layer0[key])
       symbols.setdefault(sym, []).append(cls_name)
     symbols.update({
         f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention'],
-        f'tmx::head_kernel<{min(mt, 2)}>': ['head_sample'],  # 65..128 rows: two launches of the 64-row kernel
+        ('tmx::head_wide_kernel' if batch > 128 and top_p >= 1.0 else f'tmx::head_kernel<{min(mt, 2)}>'): ['head_sample'],
+        # (65..128 rows: two launches of the 64-row kernel)
     })
     idx = {n: i for i, n in enumerate(CLASS_NAMES)}
     # An event pair around a launch also times the packet processing on both sides of it, so it
