@@ -156,9 +156,9 @@ def main():
   sampler.eos_ids = np.array([-1])  # unreachable: every row runs the full length
   rng = np.random.default_rng(0)
   # GRPO workloads: G = 8 samples of a prompt are consecutive rows; the others: distinct prompts
-  n_prompts = max(batch // 8, 1) if 'grpo' in args.workload else batch
+  n_prompts = max((batch + 7) // 8, 1) if 'grpo' in args.workload else batch
   base = rng.integers(3, cfg.vocab_size, (n_prompts, prompt)).astype(np.int32)
-  ids = np.repeat(base, batch // n_prompts, axis=0)  # G samples of a prompt are consecutive rows
+  ids = np.repeat(base, -(-batch // n_prompts), axis=0)[:batch]  # G samples of a prompt are consecutive rows
 
   walk_ms = []
 

@@ -190,6 +190,11 @@ class Sampler:
 
   def _c_state(self, st, tokens_per_pass=1):
     b, total = st['token_buffer'].shape
+    rows = b * max(tokens_per_pass, 1)
+    if rows > 128 and (rows > 4096 or not self._many_rows_ok()):
+      raise ValueError(
+          f'{b} sequences x {max(tokens_per_pass, 1)} tokens per pass: at most 4096 rows for dense models whose '
+          'projections all have K % 128 == 0, at most 128 rows otherwise (MoE models)')
     ws_bytes = self._lib.tmx_decode_workspace_bytes(
         ctypes.byref(self._transformer.desc()), b * tokens_per_pass, self.cache_config.cache_size)
     if self._workspace is None or self._workspace.numel() < ws_bytes:
@@ -224,11 +229,15 @@ class Sampler:
   MAX_ROWS = 128        # rows of one pass that chooses tokens (sequences x tokens per pass)
   MAX_FILL_ROWS = 4096  # rows of one cache-fill or scoring pass of a dense model (256-row projection blocks)
 
-  def _fill_rows(self):
+  def _many_rows_ok(self):
+    """More than 128 rows per pass need the 256-row projection blocks: a dense model whose
+    projections all have K % 128 == 0."""
     cfg = self._transformer.config
     ks = (cfg.embed_dim, cfg.num_heads * cfg.head_dim, cfg.hidden_dim)
-    wide = not cfg.num_experts and all(k % 128 == 0 for k in ks)
-    return self.MAX_FILL_ROWS if wide else self.MAX_ROWS
+    return not cfg.num_experts and all(k % 128 == 0 for k in ks)
+
+  def _fill_rows(self):
+    return self.MAX_FILL_ROWS if self._many_rows_ok() else self.MAX_ROWS
 
   def walk(self, st, n_tokens, sample=False):
     """Advances every sequence by n_tokens known tokens (cache fill over a prompt, or scoring
