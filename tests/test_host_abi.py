@@ -92,6 +92,25 @@ def test_sampler_rejects_invalid_inputs_like_the_reference():
     _sampler(8)(input_strings=['3 4 5 6 7'], max_generation_steps=4, max_prompt_length=8)
 
 
+def test_sampler_row_limits_are_checked_on_the_host():
+  """More than 128 rows per pass need a dense model with K % 128 == 0 everywhere; 4096 rows at most."""
+  import dataclasses
+  import torch
+  s = _sampler(16)
+  assert s._many_rows_ok() and s._fill_rows() == s.MAX_FILL_ROWS
+  st = {'token_buffer': torch.zeros(5000, 16, dtype=torch.int32)}
+  with pytest.raises(ValueError, match='at most 4096 rows'):
+    s._c_state(st)
+  moe = _sampler(16)
+  moe._transformer.config = dataclasses.replace(ModelConfig.toy(), num_experts=8, num_experts_per_tok=2)
+  assert not moe._many_rows_ok() and moe._fill_rows() == moe.MAX_ROWS
+  with pytest.raises(ValueError, match='at most 128 rows otherwise'):
+    moe._c_state({'token_buffer': torch.zeros(130, 16, dtype=torch.int32)})
+  odd = _sampler(16)
+  odd._transformer.config = dataclasses.replace(ModelConfig.toy(), hidden_dim=ModelConfig.toy().hidden_dim + 64)
+  assert not odd._many_rows_ok()
+
+
 def test_sampler_tokenize_and_surface():
   s = _sampler(16)
   np.testing.assert_array_equal(s.tokenize('5 6 7'), [1, 5, 6, 7])  # bos prepended
