@@ -45,6 +45,7 @@ extern "C" {
 #define TMX_MAX_RPAD 128   /* widest padded LoRA projection (sum of fused ranks, rounded up to 32) */
 #define TMX_MAX_SPLITS 16  /* most K-slices a projection is split into */
 #define TMX_MAX_LORA_SPLITS 32 /* most K-slices of the LoRA projection x . A */
+#define TMX_MAX_MOE_PAIRS 8192 /* most routed (token, expert) pairs of one pass: rows x experts_per_tok */
 #define TMX_MAX_FILL_ROWS 4096 /* most rows (sequences x tokens per sequence) of one pass of tmx_decode_steps */
 
 #define TMX_SAMPLE_GREEDY 0
@@ -204,7 +205,7 @@ int tmx_moe_route(void* stream, const void* x, const void* router_w, int B, int 
  *   down == 0: x = hidden states [P / top_k, K = D] (row p / top_k), N = 2 F with columns
  *              gate | up; out[p, 0:F] = bf16(silu(gate) * up) (F % 64 == 0)
  *   down != 0: x = activations [P, K = F] (row p); out[p, 0:N] = bf16(x . W_e) (N % 128 == 0)
- * K % 256 == 0, P <= 1024. */
+ * K % 256 == 0, P <= TMX_MAX_MOE_PAIRS. */
 int tmx_moe_experts(void* stream, const void* x, int ldx, const void* qweight, const void* scales,
                     const int32_t* expert_of, int P, int top_k, int E, int K, int N, int G, int down,
                     void* out, int ldo);
@@ -273,9 +274,9 @@ typedef struct {
                               sample == 0, or TMX_SAMPLE_SCORE): every pass consumes the T tokens at
                               columns *step .. *step + T - 1 of each sequence as batch * T rows, each
                               attending to the slots up to its own column; *step advances by T.
-                              Rows of a pass (batch * T, also for T <= 1): <= 128 for MoE models; a
-                              dense model takes up to TMX_MAX_FILL_ROWS when every projection has
-                              K % 128 == 0.
+                              Rows of a pass (batch * T, also for T <= 1): up to TMX_MAX_FILL_ROWS when
+                              every projection has K % 128 == 0 (MoE models: rows * experts_per_tok <=
+                              TMX_MAX_MOE_PAIRS), else 128.
                               The workspace must be sized for batch * T rows. */
 } tmx_decode_state;
 

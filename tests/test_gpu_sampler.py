@@ -430,8 +430,8 @@ def test_multi_token_passes_equal_one_token_passes(family):
   s = _sampler(model, cfg, 64)
   s.eos_ids = np.array([-1])
   rng = np.random.default_rng(3)
-  # dense models: 8 sequences, so that 40 tokens per pass are 320 rows (256-row projection blocks)
-  ids = rng.integers(3, cfg.vocab_size, (3 if family == 'moe' else 8, 41)).astype(np.int32)
+  # 8 sequences, so that 40 tokens per pass are 320 rows (256-row projection blocks; MoE: 640 routed pairs)
+  ids = rng.integers(3, cfg.vocab_size, (8, 41)).astype(np.int32)
   ids[1, :7] = 0   # left padding
   ids[2, :1] = 0
   def fill(tokens_per_pass):
@@ -458,7 +458,8 @@ def test_multi_token_passes_equal_one_token_passes(family):
     one = s.per_token_logps(prompt, comp, pad_id=0)
   finally:
     s.MAX_ROWS, s.MAX_FILL_ROWS = Sampler.MAX_ROWS, Sampler.MAX_FILL_ROWS
-  assert np.abs(got - one).max() <= LOGPROB_TOL, np.abs(got - one).max()
+  # (MoE: a rounding flip of a hidden state near a routing tie changes an expert weight, hence twice the slack)
+  assert np.abs(got - one).max() <= (2 if family == 'moe' else 1) * LOGPROB_TOL, np.abs(got - one).max()
   with pytest.raises(Exception):
     s.run_steps(s.init_sample_state(ids, 48, False, None, 0.0, None, None, 0), 1, sample=True, tokens_per_pass=2)
 

@@ -93,22 +93,24 @@ def test_sampler_rejects_invalid_inputs_like_the_reference():
 
 
 def test_sampler_row_limits_are_checked_on_the_host():
-  """More than 128 rows per pass need a dense model with K % 128 == 0 everywhere; 4096 rows at most."""
+  """More than 128 rows per pass need K % 128 == 0 in every projection; 4096 rows at most; MoE models
+  at most 8192 routed pairs per pass."""
   import dataclasses
   import torch
   s = _sampler(16)
   assert s._many_rows_ok() and s._fill_rows() == s.MAX_FILL_ROWS
-  st = {'token_buffer': torch.zeros(5000, 16, dtype=torch.int32)}
   with pytest.raises(ValueError, match='at most 4096 rows'):
-    s._c_state(st)
+    s._c_state({'token_buffer': torch.zeros(5000, 16, dtype=torch.int32)})
   moe = _sampler(16)
-  moe._transformer.config = dataclasses.replace(ModelConfig.toy(), num_experts=8, num_experts_per_tok=2)
-  assert not moe._many_rows_ok() and moe._fill_rows() == moe.MAX_ROWS
-  with pytest.raises(ValueError, match='at most 128 rows otherwise'):
-    moe._c_state({'token_buffer': torch.zeros(130, 16, dtype=torch.int32)})
+  moe._transformer.config = dataclasses.replace(ModelConfig.toy(), num_experts=16, num_experts_per_tok=8)
+  assert moe._max_rows() == 1024 and moe._fill_rows() == 1024
+  with pytest.raises(ValueError, match='at most 1024 rows'):
+    moe._c_state({'token_buffer': torch.zeros(1025, 16, dtype=torch.int32)})
   odd = _sampler(16)
   odd._transformer.config = dataclasses.replace(ModelConfig.toy(), hidden_dim=ModelConfig.toy().hidden_dim + 64)
-  assert not odd._many_rows_ok()
+  assert not odd._many_rows_ok() and odd._fill_rows() == 128
+  with pytest.raises(ValueError, match='at most 128 rows'):
+    odd._c_state({'token_buffer': torch.zeros(130, 16, dtype=torch.int32)})
 
 
 def test_sampler_tokenize_and_surface():

@@ -127,11 +127,11 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   if (T > 1 && sample && s->sampling_mode != TMX_SAMPLE_SCORE) return TMX_ERR_ARG;
   const int B = NSEQ * T, C = s->cache_size, L = s->buf_len;
   // a pass takes up to TMX_MAX_FILL_ROWS rows; above 128 rows the projections multiply in 256-row
-  // blocks (dense models, every K % 128 == 0), the head takes its rows 64 at a time (scoring: 256 x 256
-  // blocks); MoE models stay at 128 rows
-  if (B > (moe ? 128 : TMX_MAX_FILL_ROWS) || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
+  // blocks (every K % 128 == 0), the head takes its rows 64 at a time or in 256 x 256 blocks; MoE models
+  // are bounded by the routed pairs per pass (checked below)
+  if (B > TMX_MAX_FILL_ROWS || C <= 0 || L <= 0 || L > C) return TMX_ERR_SHAPE;
   if (moe && (m->experts_per_tok <= 0 || m->experts_per_tok > m->num_experts ||
-              (size_t)B * m->experts_per_tok > 1024))
+              (size_t)B * m->experts_per_tok > TMX_MAX_MOE_PAIRS))
     return TMX_ERR_SHAPE;
   const bool nucleus = sample && s->sampling_mode == TMX_SAMPLE_TOP_P && (s->top_p < 1.0f || s->top_k > 0);
   if (nucleus && !s->nucleus_workspace) return TMX_ERR_ARG;

@@ -355,7 +355,7 @@ constexpr int kMoeRing = 4;  // divides K / 64 (K % 256 == 0), so a ring slot is
 
 template <bool DOWN>
 __global__ __launch_bounds__(256, 2) void moe_stream_kernel(MoeArgs m) {
-  __shared__ int rows_s[1024];
+  __shared__ int rows_s[TMX_MAX_MOE_PAIRS];
   __shared__ int wave_cnt[4];
   __shared__ int n_s;
   constexpr int TPU = DOWN ? 1 : 2;  // tiles per unit: one column tile, or a gate tile and its up tile
@@ -363,9 +363,11 @@ __global__ __launch_bounds__(256, 2) void moe_stream_kernel(MoeArgs m) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, nl = lane & 31;
   int base = 0;
+  int ev = tid < m.P ? m.expert_of[tid] : -1;
   for (int p0 = 0; p0 < m.P; p0 += 256) {  // ordered compaction of { p : expert_of[p] == e }
     const int p = p0 + tid;
-    const bool hit = p < m.P && m.expert_of[p] == e;
+    const bool hit = ev == e;
+    ev = p + 256 < m.P ? m.expert_of[p + 256] : -1;  // the next round's entry travels during this one's barriers
     const unsigned long long mask = __ballot(hit);
     if (lane == 0) wave_cnt[wave] = __popcll(mask);
     __syncthreads();
@@ -468,7 +470,7 @@ __global__ __launch_bounds__(256, 2) void moe_stream_kernel(MoeArgs m) {
 
 int moe_experts(hipStream_t st, const MoeArgs& a, int E, bool down) {
   if (!a.x || !a.qw || !a.scales || !a.expert_of || !a.out) return TMX_ERR_ARG;
-  if (a.P <= 0 || a.P > 1024 || a.top_k <= 0 || E <= 0) return TMX_ERR_SHAPE;
+  if (a.P <= 0 || a.P > TMX_MAX_MOE_PAIRS || a.top_k <= 0 || E <= 0) return TMX_ERR_SHAPE;
   if (a.K % 256 || a.G % 64 || (a.G & (a.G - 1)) || a.K % a.G || a.ldx % 8) return TMX_ERR_SHAPE;
   if (a.N % 128) return TMX_ERR_SHAPE;  // gate | up: F % 64 == 0
   // decode: few rows per expert, a pure weight stream

@@ -191,10 +191,10 @@ class Sampler:
   def _c_state(self, st, tokens_per_pass=1):
     b, total = st['token_buffer'].shape
     rows = b * max(tokens_per_pass, 1)
-    if rows > 128 and (rows > 4096 or not self._many_rows_ok()):
+    if rows > self._max_rows():
       raise ValueError(
-          f'{b} sequences x {max(tokens_per_pass, 1)} tokens per pass: at most 4096 rows for dense models whose '
-          'projections all have K % 128 == 0, at most 128 rows otherwise (MoE models)')
+          f'{b} sequences x {max(tokens_per_pass, 1)} tokens per pass: this model takes at most {self._max_rows()} rows '
+          '(4096 when every projection has K % 128 == 0, MoE models 8192 / experts per token, else 128)')
     ws_bytes = self._lib.tmx_decode_workspace_bytes(
         ctypes.byref(self._transformer.desc()), b * tokens_per_pass, self.cache_config.cache_size)
     if self._workspace is None or self._workspace.numel() < ws_bytes:
@@ -229,15 +229,24 @@ class Sampler:
   MAX_ROWS = 128        # rows of one pass that chooses tokens (sequences x tokens per pass)
   MAX_FILL_ROWS = 4096  # rows of one cache-fill or scoring pass of a dense model (256-row projection blocks)
 
-  def _many_rows_ok(self):
-    """More than 128 rows per pass need the 256-row projection blocks: a dense model whose
-    projections all have K % 128 == 0."""
+  MAX_MOE_PAIRS = 8192  # routed (token, expert) pairs of one pass of a MoE model
+
+  def _max_rows(self):
+    """Rows one pass can take: more than 128 need the 256-row projection blocks (every attention /
+    dense-MLP projection with K % 128 == 0); MoE models are bounded by the routed pairs per pass."""
     cfg = self._transformer.config
-    ks = (cfg.embed_dim, cfg.num_heads * cfg.head_dim, cfg.hidden_dim)
-    return not cfg.num_experts and all(k % 128 == 0 for k in ks)
+    ks = [cfg.embed_dim, cfg.num_heads * cfg.head_dim] + ([] if cfg.num_experts else [cfg.hidden_dim])
+    if not all(k % 128 == 0 for k in ks):
+      return 128
+    if cfg.num_experts:
+      return max(128, min(4096, self.MAX_MOE_PAIRS // cfg.num_experts_per_tok))
+    return 4096
+
+  def _many_rows_ok(self):
+    return self._max_rows() > 128
 
   def _fill_rows(self):
-    return self.MAX_FILL_ROWS if self._many_rows_ok() else self.MAX_ROWS
+    return max(self.MAX_ROWS, min(self.MAX_FILL_ROWS, self._max_rows()))
 
   def walk(self, st, n_tokens, sample=False):
     """Advances every sequence by n_tokens known tokens (cache fill over a prompt, or scoring
