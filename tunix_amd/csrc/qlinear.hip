@@ -468,11 +468,77 @@ __global__ __launch_bounds__(256, 2) void moe_stream_kernel(MoeArgs m) {
   }
 }
 
+// Many rows per expert (cache fill and scoring passes of a MoE model: thousands of routed pairs): the
+// stream kernel above would re-read the gathered activation rows in every wave, so here a workgroup
+// (column block, expert) runs the 4-wave block over the expert's rows in chunks of 32 with the
+// activation slab shared in LDS (gathered rows in, scattered rows out).  DOWN = false fuses SwiGLU: the
+// workgroup owns 64 gate columns and the matching 64 up columns.
+template <bool DOWN>
+__global__ __launch_bounds__(256, 2) void moe_block_kernel(MoeArgs m) {
+  __shared__ __align__(16) uint16_t xs[2][32][kXStride];
+  __shared__ int rows_s[TMX_MAX_MOE_PAIRS];
+  __shared__ int src_s[32], dst_s[32];
+  __shared__ int wave_cnt[4];
+  __shared__ int n_s;
+  const int e = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int base = 0;
+  int ev = tid < m.P ? m.expert_of[tid] : -1;
+  for (int p0 = 0; p0 < m.P; p0 += 256) {  // ordered compaction of { p : expert_of[p] == e }
+    const int p = p0 + tid;
+    const bool hit = ev == e;
+    ev = p + 256 < m.P ? m.expert_of[p + 256] : -1;  // the next round's entry travels during this one's barriers
+    const unsigned long long mask = __ballot(hit);
+    if (lane == 0) wave_cnt[wave] = __popcll(mask);
+    __syncthreads();
+    int off = base;
+    for (int w = 0; w < wave; ++w) off += wave_cnt[w];
+    if (hit) rows_s[off + __popcll(mask & ((1ull << lane) - 1ull))] = p;
+    base += wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
+    __syncthreads();
+  }
+  if (tid == 0) n_s = base;
+  __syncthreads();
+  const int n = n_s;
+  if (n == 0) return;
+  QLinearArgs a = {};
+  a.x = m.x;
+  a.ldx = m.ldx;
+  a.qw = m.qw + (size_t)e * m.qw_stride;
+  a.scales = m.scales + (size_t)e * m.sc_stride;
+  a.y_bf16 = m.out;
+  a.ldy = m.ldo;
+  a.K = m.K; a.N = m.N; a.G = m.G;
+  a.n_main_blocks = gridDim.x;
+  a.nsplit = 1;
+  a.kt_per_split = m.K >> 6;
+  a.fixed_slice = 0;
+  a.row_src = src_s;
+  a.row_dst = dst_s;
+  a.pair_off = DOWN ? 0 : (m.N >> 6);  // tiles in F = N / 2 columns
+  for (int c0 = 0; c0 < n; c0 += 32) {
+    if (tid < 32 && c0 + tid < n) {
+      const int p = rows_s[c0 + tid];
+      src_s[tid] = DOWN ? p : p / m.top_k;
+      dst_s[tid] = p;
+    }
+    __syncthreads();
+    a.M = n - c0 < 32 ? n - c0 : 32;
+    gemm_block4<1, false>(a, xs);
+    __syncthreads();
+  }
+}
+
+
 int moe_experts(hipStream_t st, const MoeArgs& a, int E, bool down) {
   if (!a.x || !a.qw || !a.scales || !a.expert_of || !a.out) return TMX_ERR_ARG;
   if (a.P <= 0 || a.P > TMX_MAX_MOE_PAIRS || a.top_k <= 0 || E <= 0) return TMX_ERR_SHAPE;
   if (a.K % 256 || a.G % 64 || (a.G & (a.G - 1)) || a.K % a.G || a.ldx % 8) return TMX_ERR_SHAPE;
   if (a.N % 128) return TMX_ERR_SHAPE;  // gate | up: F % 64 == 0
+  if (a.P > 1024) {  // many rows per expert: the block kernel with the activation slab in LDS
+    if (down) hipLaunchKernelGGL(moe_block_kernel<true>, dim3(a.N / 128, E), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(moe_block_kernel<false>, dim3(a.N / 128, E), dim3(256), 0, st, a);
+    return check_launch();
+  }
   // decode: few rows per expert, a pure weight stream
   // column groups per expert: one gate | up pair (2 x K / 64 weight tiles) or two down tiles per wave
   // (measured on the 30B-A3B shapes: 6 groups for gate | up, 8 for down; fewer leave CUs short of
