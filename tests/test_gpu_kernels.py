@@ -585,7 +585,10 @@ def test_moe_route_matches_oracle(B, D, E, k):
   assert all(len(set(r)) == k for r in got_idx)
 
 
-@pytest.mark.parametrize('B,D,F,E,k,group', [(8, 256, 256, 16, 4, 64), (32, 512, 256, 32, 8, 128), (40, 256, 512, 4, 2, 64)])
+@pytest.mark.parametrize('B,D,F,E,k,group', [
+    (8, 256, 256, 16, 4, 64), (32, 512, 256, 32, 8, 128), (40, 256, 512, 4, 2, 64),
+    # more than 1024 routed pairs (many-rows passes): the block kernel, hundreds of rows per expert
+    (600, 256, 256, 6, 2, 64), (300, 512, 256, 9, 4, 128)])
 def test_moe_experts_match_oracle(B, D, F, E, k, group):
   T = G.Keep()
   rng = np.random.default_rng(B * 3 + E)
@@ -620,7 +623,11 @@ def test_moe_experts_match_oracle(B, D, F, E, k, group):
     g, u = lin(gate[e])(xe, BF16), lin(up[e])(xe, BF16)
     want_act = bf16_round(L.silu(g, BF16) * u)
     # a one-ulp flip of g or u (f32 accumulation order) moves the product by about one ulp of it
-    G.assert_bf16_close(got_act[rows], want_act, ulps=2.0, extra=1e-6, min_exact=0.98, what=f'act e{e}')
-    want_y = lin(down[e])(got_act[rows], BF16)  # the kernel's own activations: isolates the down product
-    G.assert_bf16_close(got_y[rows], want_y, ulps=1.0, min_exact=0.995, what=f'down e{e}')
+    few = 2 if rows.size > 128 else 0  # hundreds of thousands of outputs: sums that cancel to far below their terms
+    G.assert_bf16_close(got_act[rows], want_act, ulps=2.0, extra=1e-6, min_exact=0.98, what=f'act e{e}', stragglers=few)
+    ld = lin(down[e])
+    want_y = ld(got_act[rows], BF16)  # the kernel's own activations: isolates the down product
+    # sums that cancel to far below their terms carry the f32 accumulation error itself (eps32 x sum |x w|)
+    acc_err = 2.0 ** -23 * (np.abs(got_act[rows]) @ np.abs(ld.weight()))
+    G.assert_bf16_close(got_y[rows], want_y, ulps=1.0, extra=acc_err, min_exact=0.995, what=f'down e{e}', stragglers=few)
   assert not np.isin(idx, E - 1).any()
