@@ -588,7 +588,7 @@ def test_moe_route_matches_oracle(B, D, E, k):
 @pytest.mark.parametrize('B,D,F,E,k,group', [
     (8, 256, 256, 16, 4, 64), (32, 512, 256, 32, 8, 128), (40, 256, 512, 4, 2, 64),
     # more than 1024 routed pairs (many-rows passes): the block kernel, hundreds of rows per expert
-    (600, 256, 256, 6, 2, 64), (300, 512, 256, 9, 4, 128)])
+    (600, 256, 256, 6, 2, 64), (300, 512, 256, 9, 4, 128), (300, 256, 256, 40, 4, 64)])
 def test_moe_experts_match_oracle(B, D, F, E, k, group):
   T = G.Keep()
   rng = np.random.default_rng(B * 3 + E)
