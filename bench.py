@@ -109,6 +109,9 @@ def main():
   ap.add_argument('--workload', default='llama3.1-8b-grpo', choices=sorted(WORKLOADS))
   ap.add_argument('--sequences', type=int, default=0,
                   help='override the number of sequences of the workload (the headline metric is the default)')
+  ap.add_argument('--scoring', action='store_true',
+                  help='time the scoring pass instead (Sampler.per_token_logps over prompt + new tokens of every '
+                       'sequence): a separate JSON line, not the headline metric')
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--no-profile', action='store_true')
   ap.add_argument('--graph', action='store_true', help='replay one recorded decode step (tmx_decode_steps_graph)')
@@ -159,6 +162,30 @@ def main():
   n_prompts = max((batch + 7) // 8, 1) if 'grpo' in args.workload else batch
   base = rng.integers(3, cfg.vocab_size, (n_prompts, prompt)).astype(np.int32)
   ids = np.repeat(base, -(-batch // n_prompts), axis=0)[:batch]  # G samples of a prompt are consecutive rows
+
+  if args.scoring:
+    # Teacher forcing over whole sequences (tunix/rl/common.py:426-606): prompt cache fill + scored completion.
+    comp = rng.integers(3, cfg.vocab_size, (batch, new)).astype(np.int32)
+    times = []
+    for _ in range(3):
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      lp = sampler.per_token_logps(ids, comp, pad_id=0, temperature=1.0)
+      torch.cuda.synchronize()
+      times.append(time.perf_counter() - t0)
+    assert lp.shape == (batch, new) and np.isfinite(lp).all() and (lp <= 0).all()
+    dt = min(times[1:])
+    print(json.dumps({
+        'metric': 'scored tokens/s at 1 GPU, int4 QLoRA scoring pass (per-token log-probs)',
+        'value': batch * (prompt + new) / dt, 'unit': 'tokens/s', 'n_gpus': 1, 'ms_per_pass': dt * 1e3,
+        'higher_is_better': True, 'vs_baseline': None,
+        'dtype': 'bf16 activations / int4 weights / f32 accumulate',
+        'data': 'synthetic (random-init weights, uniform-random token ids)',
+        'config': {'workload': args.workload, 'shape': name, 'sequences': batch, 'prompt_len': prompt,
+                   'scored_tokens': new, 'quant': f'int4 group {group}', 'lora_rank': rank,
+                   'rows_per_pass': min(sampler._fill_rows() // batch, 128) * batch},
+    }))
+    return
 
   walk_ms = []
 
