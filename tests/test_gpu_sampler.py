@@ -342,19 +342,21 @@ def test_moe_decoder_matches_oracle():
   _compare_greedy(out, ref, 4, min_checked=20, lp_extra=2.0 ** -7)
 
 
-def test_graph_replay_matches_plain_launches_on_every_replay():
+@pytest.mark.parametrize('nseq', [4, 150])
+def test_graph_replay_matches_plain_launches_on_every_replay(nseq):
   """tmx_decode_steps_graph against tmx_decode_steps: several graph calls in a row, with the
   program's own eager work (a plain step, host reads) and synchronisation between them; every
-  call's tokens, logprobs, KV cache and step counter equal the plain launches'."""
+  call's tokens, logprobs, KV cache and step counter equal the plain launches'.  150 sequences:
+  the launches of the many-rows kernels are recorded."""
   cfg = C.TOY
   _, model = _pair(cfg, seed=17, targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
   rng = np.random.default_rng(2)
-  ids = np.stack([rng.integers(3, cfg.vocab_size, 8) for _ in range(4)]).astype(np.int32)
+  ids = np.stack([rng.integers(3, cfg.vocab_size, 8) for _ in range(nseq)]).astype(np.int32)
   def run(graph):
     s = _sampler(model, cfg, 64)
     s.eos_ids = np.array([-1])
     st = s.init_sample_state(ids, 64, False, None, 0.9, 1.0, None, 5, include_logprobs=True,
-                             prompt_lengths=np.full(4, 8))
+                             prompt_lengths=np.full(nseq, 8))
     snaps = []
     s.run_steps(st, 7, sample=False, graph=graph)
     for n in (9, 1, 12, 5, 16):
