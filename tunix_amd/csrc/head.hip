@@ -284,6 +284,7 @@ struct HW {
   static constexpr size_t LDS = (size_t)2 * ROWS * XS * 2;  // 128 KiB
 };
 
+template <int MODE>  // TMX_SAMPLE_*: the epilogue is compiled per mode
 __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_blocks, int voc_blocks) {
   extern __shared__ __align__(16) uint16_t smem[];
   constexpr int MT = HW::MT, TS = HW::TS, XS = HW::XS, ROWS = HW::ROWS;
@@ -376,7 +377,7 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
   // per sequence row: running max and sum of exp over this block's vocabulary rows and the best
   // candidate by key, as in head_kernel: greedy key = logit; sampling key = z + Gumbel noise of the
   // counter row * V + v; scoring: the given next token (key 0 marks it)
-  const bool score = a.mode == TMX_SAMPLE_SCORE, sampling = a.mode == TMX_SAMPLE_TOP_P;
+  constexpr bool score = MODE == TMX_SAMPLE_SCORE, sampling = MODE == TMX_SAMPLE_TOP_P;
   uint32_t key0 = 0, key1 = 0;
   if (sampling) threefry2x32(a.k0, a.k1, 0u, (uint32_t)*a.step, key0, key1);
   const int tpp = a.tpp > 0 ? a.tpp : 1;
@@ -406,8 +407,12 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
       } else {
         se += expf(z - mx);
       }
-      Best c = {key, z, v};
-      best_merge(best, c);
+      if (score) {
+        if (v == target) best = {0.f, z, v};  // at most one vocabulary row is the target
+      } else {
+        Best c = {key, z, v};
+        best_merge(best, c);
+      }
   });
   {
     const float mx2 = __shfl_xor(mx, 32, 64), se2 = __shfl_xor(se, 32, 64);
@@ -424,17 +429,27 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
 
 // M rows (any count) with the wide kernel + the finalize kernel: greedy, sampling without the sorting
 // branch, or scoring; the caller has checked: no forbidden ids, no logits output, D % 128 == 0.
+template <int MODE>
+static int launch_head_wide(hipStream_t st, const HeadArgs& a, int tok_blocks, int voc_blocks) {
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&head_wide_kernel<MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)HW::LDS);
+  if (attr != hipSuccess) return TMX_ERR_LAUNCH;
+  hipLaunchKernelGGL(head_wide_kernel<MODE>, dim3(tok_blocks * voc_blocks), dim3(512), HW::LDS, st, a, tok_blocks,
+                     voc_blocks);
+  return TMX_OK;
+}
+
 int head_wide(hipStream_t st, HeadArgs a) {
   if (a.D % 128 || a.M <= 0 || (size_t)a.M * a.D * 2 >= (1u << 31) || (size_t)256 * a.D * 2 >= (1u << 31))
     return TMX_ERR_SHAPE;
-  static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&head_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)HW::LDS);
-  if (attr != hipSuccess) return TMX_ERR_LAUNCH;
   const int tok_blocks = (a.M + 255) / 256, voc_blocks = (a.V + HW::ROWS - 1) / HW::ROWS;
   a.nwg = voc_blocks;
   a.row_base = 0;
-  hipLaunchKernelGGL(head_wide_kernel, dim3(tok_blocks * voc_blocks), dim3(512), HW::LDS, st, a, tok_blocks,
-                     voc_blocks);
+  int lrc;
+  if (a.mode == TMX_SAMPLE_SCORE) lrc = launch_head_wide<TMX_SAMPLE_SCORE>(st, a, tok_blocks, voc_blocks);
+  else if (a.mode == TMX_SAMPLE_TOP_P) lrc = launch_head_wide<TMX_SAMPLE_TOP_P>(st, a, tok_blocks, voc_blocks);
+  else lrc = launch_head_wide<TMX_SAMPLE_GREEDY>(st, a, tok_blocks, voc_blocks);
+  if (lrc != TMX_OK) return lrc;
   int rc = check_launch();
   if (rc != TMX_OK) return rc;
   hipLaunchKernelGGL(head_finalize_kernel, dim3(a.M), dim3(256), 0, st, a);
