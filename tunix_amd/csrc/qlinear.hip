@@ -1450,9 +1450,13 @@ __global__ __launch_bounds__(512, 1) void qlinear_mfma_wide_kernel(QLinearArgs a
   const int id = (int)blockIdx.x, xcd = id & 7, idx = id >> 3;
   const int per_rb = blocks * a.nsplit;
   const int p = xcd / S + (8 / S) * idx;
-  const int bz = xcd % S + S * (p / per_rb);
+  // an XCD with an even number of row blocks takes them two at a time, the same column block on both in
+  // consecutive workgroups, so that a weight tile fetched for one is an L2 hit for the other
+  const int R = (row_blocks + S - 1) / S, Gr = (R & 1) ? 1 : 2;
+  const int blk = p / (per_rb * Gr), within = p % (per_rb * Gr);
+  const int bz = xcd % S + S * (blk * Gr + within % Gr);
   if (bz >= row_blocks) return;
-  const int cb = p % per_rb, bx = cb % blocks, by = cb / blocks;
+  const int cb = within / Gr, bx = cb % blocks, by = cb / blocks;
   if (bx >= a.n_main_blocks) gemm_block_wide<true>(a, smem, bx, by, bz);
   else gemm_block_wide<false>(a, smem, bx, by, bz);
 }
