@@ -88,6 +88,18 @@ def test_threefry2x32_known_answers():
     assert (int(x0), int(x1)) == tuple(num(v) for v in case['expected'])
 
 
+def test_threefry_matches_the_key_pair_of_jax_split():
+  """jax.random.split(jax.random.PRNGKey(0)) prints [[4146024105, 967050713], [2718843009, 1272950319]]
+  in JAX's own documentation (the pseudo-random numbers tutorial).  split hashes the counters
+  0..3 under the key (0, 0) with the first half as word 0 and the second half as word 1, so
+  the pair pins how JAX feeds keys and counters to threefry2x32, which fold_in shares."""
+  k0, k1 = prng.prng_key(0)
+  assert (int(k0), int(k1)) == (0, 0)
+  y0, y1 = prng.threefry2x32(k0, k1, np.array([0, 1], np.uint32), np.array([2, 3], np.uint32))
+  assert [int(v) for v in y0] == [4146024105, 967050713]
+  assert [int(v) for v in y1] == [2718843009, 1272950319]
+
+
 def test_uniform_and_gumbel_ranges():
   bits = np.array([0, 1, 0xFFFFFFFF, 0x80000000], np.uint32)
   u = prng.uniform_from_bits(bits)
