@@ -3,13 +3,17 @@
 Reference: tunix/generate/sampler.py:562 (``jax.random.fold_in(seed,
 decoding_step)``), :128 and :144 (``jax.random.categorical``), :938-941
 (``PRNGKey(0)`` default).  JAX is a third-party dependency that is not
-installed here (jax>=0.6.0, pyproject.toml:33); its published algorithm is
+installed here (jax>=0.6.0, pyproject.toml:31); its published algorithm is
 restated: threefry2x32 (Salmon et al., Random123, 20 rounds), the
 "partitionable" bit generation that is the default from jax 0.5 on
 (bits[i] = x0 ^ x1 of threefry(key, (hi32(i), lo32(i))) over the row-major
 linear index i), ``uniform`` = mantissa fill, ``gumbel`` = -log(-log(u)).
-The block function is pinned by the Random123 known-answer vectors; the wiring
-around it is parity unpinned.
+The block function is pinned by the Random123 known-answer vectors; the key and
+counter word order by the key pair JAX's documentation prints for
+split(PRNGKey(0)); random_bits and the mantissa fill by the documented value of
+normal(key(42)).  fold_in's counter words, gumbel's clamping at the smallest
+normal float and categorical's use of them have no published value to check
+against: for these the wiring is parity unpinned.
 """
 import numpy as np
 

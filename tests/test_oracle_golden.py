@@ -100,6 +100,28 @@ def test_threefry_matches_the_key_pair_of_jax_split():
   assert [int(v) for v in y1] == [2718843009, 1272950319]
 
 
+def test_random_bits_reproduce_the_documented_normal_of_key_42():
+  """JAX's documentation prints jax.random.normal(jax.random.key(42)) = -0.028304616 (releases
+  with jax_threefry_partitionable on by default, 0.5.0 and later: the reference needs
+  jax >= 0.6.0, pyproject.toml:31) and -0.18471177 before that.  normal() is
+  sqrt(2) * erfinv(u) with u uniform in (-1, 1) built from one 32-bit word the same way
+  uniform_from_bits builds it, so the first value pins random_bits (64-bit element index as the
+  counter words, x0 ^ x1 as the output) together with the mantissa trick; the second shows
+  that the older scheme (counter words (0, 0), first output word) is the one NOT restated."""
+  from scipy.special import erfinv
+
+  def normal_of(word):
+    f = ((np.uint32(word) >> np.uint32(9)) | np.uint32(0x3F800000)).view(np.float32) - np.float32(1.0)
+    lo, hi = np.nextafter(np.float32(-1.0), np.float32(0.0)), np.float32(1.0)
+    u = np.maximum(lo, f * (hi - lo) + lo)
+    return float(np.sqrt(2.0) * erfinv(np.float64(u)))
+
+  key = prng.prng_key(42)
+  assert abs(normal_of(prng.random_bits(key, (1,))[0]) - (-0.028304616)) < 2e-8
+  y0, _ = prng.threefry2x32(key[0], key[1], np.array([0], np.uint32), np.array([0], np.uint32))
+  assert abs(normal_of(y0[0]) - (-0.18471177)) < 1e-7
+
+
 def test_uniform_and_gumbel_ranges():
   bits = np.array([0, 1, 0xFFFFFFFF, 0x80000000], np.uint32)
   u = prng.uniform_from_bits(bits)
