@@ -120,6 +120,13 @@ def test_random_bits_reproduce_the_documented_normal_of_key_42():
   assert abs(normal_of(prng.random_bits(key, (1,))[0]) - (-0.028304616)) < 2e-8
   y0, _ = prng.threefry2x32(key[0], key[1], np.array([0], np.uint32), np.array([0], np.uint32))
   assert abs(normal_of(y0[0]) - (-0.18471177)) < 1e-7
+  # jax.random.uniform(jax.random.key(0)) prints 0.947667 with the partitionable scheme and
+  # 0.41845703 with the older one: the [0, 1) map itself, without the erfinv on top
+  key0 = prng.prng_key(0)
+  unit = lambda w: float(((np.uint32(w) >> np.uint32(9)) | np.uint32(0x3F800000)).view(np.float32) - np.float32(1.0))
+  assert abs(unit(prng.random_bits(key0, (1,))[0]) - 0.947667) < 5e-7
+  z0, _ = prng.threefry2x32(key0[0], key0[1], np.array([0], np.uint32), np.array([0], np.uint32))
+  assert abs(unit(z0[0]) - 0.41845703) < 5e-8
 
 
 def test_uniform_and_gumbel_ranges():
