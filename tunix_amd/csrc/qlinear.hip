@@ -1055,9 +1055,10 @@ static int launch_gate_up8(hipStream_t st, const QLinearArgs& a) {
 // the activation slab goes from global memory straight into LDS, so the loop has no per-lane
 // address arithmetic, no staging registers and no LDS stores.  A slab row is 512 bytes; a
 // direct-to-LDS load lands 1 KiB contiguously, i.e. two rows back to back, so rows are stored
-// unpadded and the 16-byte chunks of row r are XOR-swizzled by r % 8 instead (the global
-// address of every lane is free, so the swizzle costs nothing; fragment reads stay
-// conflict-free).  64 KiB of LDS and <= 128 registers: two workgroups = 16 waves per CU.
+// unpadded and the 16-byte chunks of row r are XOR-swizzled by r % 16 instead (the global
+// address of every lane is free, so the swizzle costs nothing).  A 16-byte LDS read serves 16
+// lanes per clock over 64 banks: 16 consecutive rows must land in 16 different chunk columns
+// for the fragment reads to stay conflict-free (a swizzle by r % 8 runs at half rate).  64 KiB of LDS and <= 128 registers: two workgroups = 16 waves per CU.
 struct KD {
   static constexpr int TS = 4, TPW = 2, XS = 256;
   static constexpr size_t lds(int MT) { return (size_t)2 * MT * 32 * XS * 2; }
@@ -1091,13 +1092,13 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
   const int wstep = LORA ? NT * 4096 : 1024;  // bytes between consecutive k-tiles
   const int sv = (nb * KG * 32 + nl) * 2;
   // slab transfer: XR loads per wave and step; load i moves rows 2 wave + 16 i (lanes 0..31)
-  // and the next one (lanes 32..63), lane l delivering chunk (l % 32) ^ (row % 8) to slot l % 32
+  // and the next one (lanes 32..63), lane l delivering chunk (l % 32) ^ (row % 16) to slot l % 32
   constexpr int XR = ROWS / 16;
   int xoff[XR];  // per-lane byte offset of the row's first step (rows past M repeat the last)
 #pragma unroll
   for (int i = 0; i < XR; ++i) {
     const int row_l = 2 * wave + 16 * i + h;
-    xoff[i] = (row_l < a.M ? row_l : a.M - 1) * a.ldx * 2 + ((nl ^ (row_l & 7)) * 16) + kb0 * 128;
+    xoff[i] = (row_l < a.M ? row_l : a.M - 1) * a.ldx * 2 + ((nl ^ (row_l & 15)) * 16) + kb0 * 128;
   }
 
   f32x16_t acc[MT];
@@ -1126,14 +1127,14 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
   };
   auto tile_math = [&](int step, int buf, auto dc, auto jc) __attribute__((always_inline)) {
     constexpr int d = decltype(dc)::value, j = decltype(jc)::value;
-    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + (kw * TPW + j) * 64 + nl * XS;
+    const uint16_t* xb = smem + (size_t)buf * ROWS * XS + kw * TPW * 64 + nl * XS;
     bf16x8_t xa[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        // chunk 2 t + h of the tile sits at slot (2 t + h) ^ (row % 8)
-        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + (((2 * t + h) ^ (nl & 7)) * 8));
+        // chunk 8 j + 2 t + h of the wave's tile pair sits at slot (8 j + 2 t + h) ^ (row % 16)
+        xa[m][t] = *reinterpret_cast<const bf16x8_t*>(xb + m * 32 * XS + (((8 * j + 2 * t + h) ^ (nl & 15)) * 8));
       }
     u32x4_t wc[WPT];
 #pragma unroll
