@@ -51,8 +51,10 @@ extern "C" {
 #define TMX_SAMPLE_GREEDY 0
 #define TMX_SAMPLE_TOP_P 1
 #define TMX_SAMPLE_SCORE 2 /* teacher forcing: no token is chosen; logprobs[m, *step + 1] =
-                              log_softmax(logits / temperature)[token_buffer[m, *step + 1]]
-                              (tunix/rl/common.py:426-606 compute_per_token_logps) */
+                              z[token_buffer[m, *step + 1]] - logsumexp(z), z = logits / temperature
+                              with NaN -> -1e9 and the rest clipped to [-1e9, 1e9], so the result is
+                              always finite (tunix/rl/common.py:426-606 compute_per_token_logps,
+                              :207-226 selective_log_softmax) */
 
 const char* tmx_status_string(int status);
 int tmx_abi_version(void);

@@ -7,7 +7,6 @@ packing and without chunking) with process_ids (:257-330) and selective_log_soft
 import numpy as np
 
 from oracle import masks
-from oracle import sampling
 
 
 def per_token_logps(model, prompt_tokens, completion_tokens, pad_id, temperature=1.0):
@@ -24,5 +23,18 @@ def per_token_logps(model, prompt_tokens, completion_tokens, pad_id, temperature
   logits = logits[:, -keep - 1:-1, :]                         # :590
   if temperature not in (0.0, 1.0):
     logits = logits / np.float32(temperature)                 # :591-592
-  logp = sampling.log_softmax(logits)
-  return np.take_along_axis(logp, ids[:, -keep:, None], axis=-1)[..., 0]
+  return selective_log_softmax(logits, ids[:, -keep:])
+
+
+def selective_log_softmax(logits, input_ids):
+  """common.py:207-226: NaN logits count as -1e9, the others are clipped to [-1e9, 1e9];
+  result = logits[ids] - logsumexp(logits), f32."""
+  x = np.asarray(logits, np.float32)
+  with np.errstate(invalid='ignore'):
+    x = np.where(np.isnan(x), np.float32(-1e9), np.clip(x, np.float32(-1e9), np.float32(1e9))).astype(np.float32)
+  # jax.nn.logsumexp: max + log(sum(exp(x - max))), all f32; the target's logit minus that
+  # (not the shifted form of log_softmax: at the clip the two differ by log(count))
+  mx = x.max(axis=-1, keepdims=True)
+  lse = (mx + np.log(np.exp(x - mx).sum(axis=-1, keepdims=True, dtype=np.float32))).astype(np.float32)
+  target = np.take_along_axis(x, np.asarray(input_ids)[..., None], axis=-1)
+  return (target - lse)[..., 0].astype(np.float32)

@@ -389,6 +389,46 @@ def test_head_greedy(M, D, V):
   assert clear.sum() == 0 or np.abs(lp[clear, step + 1] - o_lp[clear]).max() <= 1e-2
 
 
+def test_head_scoring_clips_logits_like_the_reference():
+  """TMX_SAMPLE_SCORE follows selective_log_softmax (tunix/rl/common.py:217-221): NaN logits count
+  as -1e9, the others are clipped to [-1e9, 1e9], so every score is finite.  Row 0 of x is 1e10:
+  vocabulary row 7 (+1e30) gives +inf, row 9 -inf, row 11 (alternating signs) inf - inf = NaN, and
+  most ordinary logits of that row are beyond the clip."""
+  from oracle import scoring
+  M, D, V, step, col_len = 4, 256, 1024, 2, 8
+  x, w = _head_inputs(M, D, V, 77)
+  x[0, :] = 1e10
+  w[7, :] = 1e30
+  w[9, :] = -1e30
+  w[11, :] = np.where(np.arange(D) % 2 == 0, 1e30, -1e30)
+  x, w = bf16_round(x), bf16_round(w)
+  targets = np.array([[7, 9, 11, 500], [7, 9, 11, 500], [3, 7, 100, 11], [9, 1, 2, 3]], np.int32)
+  lib = _lib.lib()
+  for col in range(4):
+    T = G.Keep()
+    ws = torch.empty(lib.tmx_head_sample_workspace_bytes(M, V), dtype=torch.uint8, device=G.DEV)
+    tok = torch.full((M, col_len), -5, dtype=torch.int32, device=G.DEV)
+    tok[:, step + 1] = torch.from_numpy(targets[:, col]).to(G.DEV)
+    lp = torch.zeros(M, col_len, dtype=torch.float32, device=G.DEV)
+    done = torch.zeros(M, dtype=torch.uint8, device=G.DEV)
+    logits = torch.empty(M, V, dtype=torch.float32, device=G.DEV)
+    G.call('tmx_head_sample', S(), T.bf(x), T.bf(w), M, D, V, 2, 0.5, 0, 0, T.i32([step]), None, 0,
+           T.i32([-1]), 1, G.p(tok), G.p(lp), G.p(done), col_len, G.p(logits), G.p(ws))
+    G.sync()
+    lg, got = logits.cpu().numpy(), lp.cpu().numpy()[:, step + 1]
+    if col == 0:
+      assert lg[0, 7] == np.inf and lg[0, 9] == -np.inf and np.isnan(lg[0, 11])
+      rest = np.delete(lg[0], [7, 9, 11])
+      assert np.isfinite(rest).all() and (np.abs(rest) > 1e9).mean() > 0.5  # most are beyond the clip
+    # exact function of the kernel's own logits
+    want = scoring.selective_log_softmax(lg / np.float32(0.5), targets[:, col])
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=2e-5)
+    np.testing.assert_array_equal(tok.cpu().numpy()[:, step + 1], targets[:, col])  # scoring chooses nothing
+  # row 0: +inf scores 0 against the normaliser 1e9 + log(count), NaN and -inf score -2e9
+  # (checked on the last column's neighbours through the closed form of the oracle pin)
+
+
 def test_head_greedy_ties_pick_first_index_and_forbidden():
   T = G.Keep()
   M, D, V = 3, 128, 1024

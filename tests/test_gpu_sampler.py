@@ -5,10 +5,12 @@ import numpy as np
 import pytest
 import torch
 
+from oracle import masks as OMK
 from oracle import model as OM
 from oracle import prng
 from oracle import sampler as OSAM
 from oracle import sampling as OS
+from oracle.bf16 import bf16_round
 from tunix_amd.configs import CacheConfig, RolloutConfig
 from tunix_amd.rollout import TmxRollout
 from tunix_amd.sampler import Sampler
@@ -412,6 +414,36 @@ def test_per_token_logps_match_oracle_and_the_rollout_logprobs():
   assert np.abs(scored - np.stack(ro.logprobs)).max() <= LOGPROB_TOL
   with pytest.raises(ValueError):
     s.per_token_logps(np.zeros((2, 0), np.int32), comp[:2])
+
+
+def test_scoring_clip_reaches_the_many_rows_head():
+  """A head scaled by 1e30 puts every logit beyond the reference's clip at +-1e9
+  (tunix/rl/common.py:217-221): a target with a positive logit then scores 1e9 - (1e9 + log n) = 0
+  in f32, one with a negative logit -2e9.  8 sequences x 22 tokens = 176 rows per pass: the
+  256 x 256 head kernel."""
+  from oracle import scoring
+  cfg = C.TOY
+  st = C.make_state(cfg, 31, 8, norm_jitter=0.05)
+  plain = OM.Decoder(cfg, C.oracle_weights(cfg, st, 64, 16.0, 8))
+  st['lm_head.w'] = bf16_round(st['lm_head.w'] * np.float32(1e30))
+  oracle = OM.Decoder(cfg, C.oracle_weights(cfg, st, 64, 16.0, 8))
+  model = C.product_model(cfg, st, 64, 16.0)
+  s = _sampler(model, cfg, 48)
+  rng = np.random.default_rng(4)
+  prompt = rng.integers(3, cfg.vocab_size, (8, 10)).astype(np.int32)
+  comp = rng.integers(3, cfg.vocab_size, (8, 12)).astype(np.int32)
+  got = s.per_token_logps(prompt, comp, pad_id=0)
+  want = scoring.per_token_logps(oracle, prompt, comp, 0)
+  assert np.isfinite(got).all() and set(np.unique(want)) <= {0.0, np.float32(-2e9)}
+  # the sign of a target logit is compared where the unscaled logit is clear of bf16 rounding
+  ids = np.concatenate([prompt, comp], 1)
+  valid = np.ones_like(ids, bool)
+  pos = OMK.build_positions_from_mask(valid)
+  base_logits, _ = plain(ids, pos, None, OMK.make_causal_attn_mask(valid, ids.shape[1]))
+  tgt = np.take_along_axis(base_logits[:, -13:-1, :], comp[..., None], -1)[..., 0]
+  clear = np.abs(tgt) > 0.05
+  assert clear.sum() > 48
+  np.testing.assert_array_equal(got[clear], want[clear])
 
 
 @pytest.mark.parametrize('family', ['llama3', 'qwen3', 'moe'])

@@ -389,4 +389,26 @@ def test_scoring_pass_reproduces_the_logprobs_of_generation():
   p = ref['padded_prompt_tokens'].shape[1]
   for b in range(2):
     for t in range(comp.shape[1]):
-      assert got[b, t] == lp[b, p + t - 1, comp[b, t]]
+      # logit - logsumexp against the shifted log-softmax: equal up to f32 rounding
+      assert abs(got[b, t] - lp[b, p + t - 1, comp[b, t]]) <= 2e-6
+
+
+def test_selective_log_softmax_clips_like_the_reference():
+  """tunix/rl/common.py:217-221: NaN -> -1e9, clip to [-1e9, 1e9], then logits[id] - logsumexp.
+  Closed form: with one +1e9 entry the normaliser is 1e9, so that entry scores 0, a NaN or -inf
+  entry -2e9 and a zero entry -1e9; without special values it is the plain log-softmax."""
+  from oracle import scoring
+  z = np.array([[np.nan, np.inf, 0.0, -np.inf, 3e9]], np.float32)
+  ids = np.arange(5)[None, :]
+  got = scoring.selective_log_softmax(np.repeat(z[:, None, :], 5, 1), ids)[0]
+  # two entries sit at +1e9 (inf and 3e9): logsumexp = f32(1e9 + log 2) = 1e9 exactly
+  np.testing.assert_array_equal(got, np.array([-2e9, 0.0, -1e9, -2e9, 0.0], np.float32))
+  assert np.isfinite(got).all()
+  rng = np.random.default_rng(0)
+  x = rng.standard_normal((3, 4, 50)).astype(np.float32) * 5
+  tok = rng.integers(0, 50, (3, 4))
+  want = np.take_along_axis(OS.log_softmax(x), tok[..., None], -1)[..., 0]
+  np.testing.assert_allclose(scoring.selective_log_softmax(x, tok), want, atol=4e-6)
+  # logsumexp form, not the shifted one: 600 entries at the clip score 1e9 - f32(1e9 + log 600) = 0
+  flat = scoring.selective_log_softmax(np.full((1, 600), 2e9, np.float32), np.array([5]))
+  assert flat[0] == 0.0

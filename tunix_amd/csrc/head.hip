@@ -28,6 +28,12 @@ template <int V>
 struct HIC { static constexpr int value = V; };
 constexpr int kHXStride = 72;  // bf16 elements per LDS row of the activation tile (64 + 8 pad)
 
+// Scoring (tunix/rl/common.py:217-221, selective_log_softmax): a NaN logit counts as -1e9 and
+// the others are clipped to [-1e9, 1e9] before the log-softmax, so the result is always finite.
+__device__ __forceinline__ float score_clip(float z) {
+  return z != z ? -1e9f : fminf(fmaxf(z, -1e9f), 1e9f);
+}
+
 // Workgroup = 4 waves x 32 vocabulary rows.  The hidden-state k-tile x[0:M, 64 kb : 64 kb + 64]
 // is fetched once per workgroup, double-buffered in LDS and shared by the waves (MFMA B
 // fragments); head rows stream HBM -> registers through a ring of 4 k-tiles per wave.  Lane
@@ -155,7 +161,7 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
         float z = logit, key = logit;
         if (score) {
           // the "best" candidate is the given next token: its z is what the log-prob needs
-          z = logit / a.temperature;
+          z = score_clip(logit / a.temperature);
           key = (v == target[m]) ? 0.f : -INFINITY;
         } else if (a.mode == TMX_SAMPLE_TOP_P) {
           z = logit / a.temperature;
@@ -253,8 +259,9 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
     if (a.mode == TMX_SAMPLE_SCORE) {  // teacher forcing: the token stays, only its log-prob is written
       const int tpp = a.tpp > 0 ? a.tpp : 1;
       const int prow = a.row_base + row;
+      // selective_log_softmax: logit - logsumexp, with logsumexp = max + log(sum exp(z - max))
       if (a.logprobs)
-        a.logprobs[(size_t)(prow / tpp) * a.buf_len + *a.step + prow % tpp + 1] = (best.z - mx) - logf(se);
+        a.logprobs[(size_t)(prow / tpp) * a.buf_len + *a.step + prow % tpp + 1] = best.z - (mx + logf(se));
       return;
     }
     const int col = *a.step + 1;
@@ -393,7 +400,7 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
       const float logit = rbf(acc[m][r]);
       float z = logit, key = logit;
       if (score) {
-        z = logit / a.temperature;
+        z = score_clip(logit / a.temperature);
         key = (v == target) ? 0.f : -INFINITY;
       } else if (sampling) {
         z = logit / a.temperature;
