@@ -23,7 +23,13 @@ whose arithmetic it restates.  Pinning status per function group:
   pyproject.toml:48, not vendored, not installed here).  It is a parameter.
 * threefry2x32 block function ........................... pinned by the
   Random123 known-answer vectors.
-* jax.random wiring around it (PRNGKey, fold_in, partitionable counters,
-  bits->uniform->gumbel) ................................ parity unpinned: JAX
-  is not installed; restated from the published algorithm.
+* JAX's key / counter word order, partitionable bit generation and the
+  bits->[0, 1) map ....................................... pinned by the values
+  JAX's documentation prints for split(PRNGKey(0)), normal(key(42)) and
+  uniform(key(0)).
+* fold_in's counter words, gumbel's clamp, categorical's use of them ... parity
+  unpinned: JAX is not installed and no published value covers them; restated
+  from the published algorithm.
+* selective_log_softmax (scoring) ........................ pinned by closed forms
+  (NaN / inf / clip cases, logsumexp form).
 """
