@@ -38,6 +38,7 @@ extern "C" {
 #define TMX_ERR_SHAPE (-2)       /* a dimension violates the kernel's tiling rules */
 #define TMX_ERR_LAUNCH (-3)      /* the HIP runtime refused the launch */
 #define TMX_ERR_UNSUPPORTED (-4) /* valid request outside what is implemented */
+#define TMX_ERR_SCRATCH (-5)     /* the request needs more scratch memory than the library's static buffer holds */
 
 #define TMX_FAMILY_LLAMA3 0
 #define TMX_FAMILY_QWEN3 1
@@ -79,6 +80,21 @@ size_t tmx_qlora_linear_workspace_bytes(int M, int K, int N);
 int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const void* scales,
                      const void* lora_a_t, const void* lora_b, const void* residual, void* y,
                      void* workspace, int M, int K, int N, int G, int r, int r_pad, float lora_scale);
+
+/* tmx_qlora_linear without a workspace argument and without any allocation.  No counterpart in
+ * the reference: it exists for callers that cannot allocate device memory around the call (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The K-slice and
+ * LoRA planes live in a static device array of TMX_STATIC_SCRATCH_BYTES that each GPU the library
+ * runs on holds until the process ends; a request whose tmx_qlora_linear_workspace_bytes(M, K, N)
+ * exceeds it returns TMX_ERR_SCRATCH and launches nothing (every decode shape of the 8B models
+ * up to 128 rows fits).  All calls on one GPU share that GPU's array: calls that overlap on one
+ * GPU (two streams, two threads) race; calls on one stream are ordered and safe.  Same results
+ * as tmx_qlora_linear, bit for bit. */
+#define TMX_STATIC_SCRATCH_BYTES (32u << 20)
+size_t tmx_qlora_linear_noalloc_max_bytes(void);
+int tmx_qlora_linear_noalloc(void* stream, const void* x, const void* qweight, const void* scales,
+                             const void* lora_a_t, const void* lora_b, const void* residual, void* y,
+                             int M, int K, int N, int G, int r, int r_pad, float lora_scale);
 
 /* The matrix product alone, for callers that fuse their own consumer: writes `nsplit` f32
  * K-slice planes y_part[nsplit][M][N] (their sum is x . dequant(W)) and, with LoRA,

@@ -17,6 +17,7 @@ SIGNATURES = {
     'tmx_abi_version': [],
     'tmx_int4_dequant': [vp, vp, vp, vp, ci, ci, ci],
     'tmx_qlora_linear': [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
+    'tmx_qlora_linear_noalloc': [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
     'tmx_qlora_linear_num_splits': [ci, ci, ci],
     'tmx_qlora_linear_num_lora_splits': [ci, ci],
     'tmx_qlora_linear_planes': [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci],
@@ -42,6 +43,7 @@ SIGNATURES = {
 SIZE_FUNCS = {
     'tmx_gqa_decode_workspace_bytes': [ci, ci, ci, ci, ci],
     'tmx_qlora_linear_workspace_bytes': [ci, ci, ci],
+    'tmx_qlora_linear_noalloc_max_bytes': [],
     'tmx_head_sample_workspace_bytes': [ci, ci],
     'tmx_nucleus_workspace_bytes': [ci, ci],
     'tmx_decode_workspace_bytes': [vp, ci, ci],

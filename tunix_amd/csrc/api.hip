@@ -8,8 +8,9 @@ extern "C" const char* tmx_status_string(int status) {
     case TMX_ERR_SHAPE: return "shape violates the kernel's tiling rules";
     case TMX_ERR_LAUNCH: return "HIP launch failed";
     case TMX_ERR_UNSUPPORTED: return "unsupported configuration";
+    case TMX_ERR_SCRATCH: return "the request needs more scratch memory than the library's static buffer holds";
     default: return "unknown status";
   }
 }
 
-extern "C" int tmx_abi_version(void) { return 2; }
+extern "C" int tmx_abi_version(void) { return 3; }

@@ -12,6 +12,8 @@
 // v_cvt_f32_ubyteN, scaled with one fma ((u - 8) * s is exact in f32) and
 // rounded pairwise to bf16 by the hardware converter, which reproduces the
 // reference's bf16 dequantised weight bit for bit before it enters the MFMA.
+#include <atomic>
+
 #include "tmx_kernels.h"
 
 namespace tmx {
@@ -1826,6 +1828,49 @@ extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight
                      (const uint16_t*)lora_b, r, lora_scale,
                      (const uint16_t*)residual, M, N);
   return check_launch();
+}
+
+// ---------------------------------------------------------------------------
+// tmx_qlora_linear for callers that may not allocate (HIP graph capture, serving loops): the
+// K-slice planes and LoRA planes live in a file-scope device array instead of a caller workspace.
+// Every GPU holds its own copy of the array at its own address; the address is looked up once per
+// device, with that device current, and host code only ever uses that pointer (the array's name
+// is a host-side stand-in, not a device address).
+constexpr size_t kStaticScratchBytes = TMX_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TMX_ERR_LAUNCH;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return TMX_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing first calls store the same address
+  }
+  *out = p;
+  return TMX_OK;
+}
+
+extern "C" size_t tmx_qlora_linear_noalloc_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int tmx_qlora_linear_noalloc(void* stream, const void* x, const void* qweight, const void* scales,
+                                        const void* lora_a_t, const void* lora_b, const void* residual,
+                                        void* y, int M, int K, int N, int G, int r, int r_pad,
+                                        float lora_scale) {
+  if (M <= 0 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
+  if (tmx_qlora_linear_workspace_bytes(M, K, N) > kStaticScratchBytes) return TMX_ERR_SCRATCH;
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != TMX_OK) return rc;
+  // every plane element a consumer reads is written by the projection launch of the same call,
+  // so nothing in the array has to start at zero
+  return tmx_qlora_linear(stream, x, qweight, scales, lora_a_t, lora_b, residual, y, ws, M, K, N, G, r, r_pad,
+                          lora_scale);
 }
 
 extern "C" int tmx_qlora_gate_up_swiglu(void* stream, const void* x, const void* qweight, const void* scales,
