@@ -3,9 +3,14 @@
 A "step" is one decode-loop iteration over the whole batch (one new token per
 sequence).  Default workload: Llama-3.1-8B shape, 64 sequences (8 prompts x 8
 samples), 256-token prompts, temperature 0.9, top-p 1.0, per-token logprobs,
-bf16 KV cache.  The timed region covers the generation steps that follow the
-warmup steps of the same rollout, so the context grows from 256 + warmup towards 767
-(mean about 512).  Prints one JSON line.
+bf16 KV cache.  The timed region is centred on the workload's mean context
+(prompt + new / 2): the default run times nearly the whole generation (context
+271 -> 767); a shorter run (--steps 20) first fills the cache up to the start of its
+window with known tokens, in multi-token passes, so it measures the same mean context.
+Prints one JSON line.
+
+  python bench.py --pmc-summary CSV COUNTER [--match TEXT]   per-kernel means of one hardware
+      counter from a rocprofv3 counter-collection CSV (how profiles/ summaries are made)
 """
 import argparse
 import ctypes
@@ -101,8 +106,28 @@ def cpu_baseline(workload, n_layers=2):
   }
 
 
+def pmc_summary(path, counter, match=None, top=16):
+  """Prints, for every kernel symbol of a rocprofv3 counter-collection CSV, the number of
+  dispatches and the mean / max of `counter` over them (template arguments kept, argument
+  lists dropped)."""
+  import collections
+  import csv
+  agg = collections.defaultdict(list)
+  with open(path) as f:
+    for row in csv.DictReader(f):
+      if row['Counter_Name'] != counter or (match and match not in row['Kernel_Name']):
+        continue
+      agg[row['Kernel_Name'].split('(')[0]].append(float(row['Counter_Value']))
+  rows = sorted(agg.items(), key=lambda kv: -sum(kv[1]))[:top]
+  for k, v in rows:
+    print(f"{counter} {k[:80]:80s} launches {len(v):7d} mean {sum(v) / len(v):14.1f} max {max(v):14.1f}")
+
+
 def main():
   ap = argparse.ArgumentParser()
+  ap.add_argument('--pmc-summary', nargs=2, metavar=('CSV', 'COUNTER'), default=None,
+                  help='summarise one counter of a rocprofv3 counter-collection CSV per kernel and exit (no GPU)')
+  ap.add_argument('--match', default=None, help='--pmc-summary: only kernels whose name contains this text')
   ap.add_argument('--gpus', type=int, default=1)
   ap.add_argument('--steps', type=int, default=496)
   ap.add_argument('--warmup', type=int, default=16)
@@ -121,6 +146,9 @@ def main():
   ap.add_argument('--pmc-calibrate', action='store_true',
                   help='also run one 1 GiB device copy (a kernel of known traffic) to scale PMC counters')
   args = ap.parse_args()
+  if args.pmc_summary:
+    pmc_summary(args.pmc_summary[0], args.pmc_summary[1], args.match)
+    return
   if args.gpus != 1:
     print('bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1',
           file=sys.stderr)
@@ -188,17 +216,23 @@ def main():
     return
 
   walk_ms = []
+  # The timed window [start + warmup, start + warmup + steps) is centred on the workload's mean
+  # context prompt + new / 2.  A run shorter than the generation stands in for its middle: the
+  # columns between the prompt and `start` hold known (random) tokens, as if already generated,
+  # and are walked by the same cache fill as the prompt.
+  start = max(prompt, prompt + (new - args.steps) // 2 - args.warmup)
+  filled = np.concatenate([ids, rng.integers(3, cfg.vocab_size, (batch, start - prompt)).astype(np.int32)], axis=1)
 
   def fresh_state():
-    st = sampler.init_sample_state(ids, prompt + new, False, None, temp, top_p, None, 0,
-                                   include_logprobs=True, prompt_lengths=np.full(batch, prompt))
-    # cache fill over the prompt (outside the timed region), in multi-token passes
+    st = sampler.init_sample_state(filled, prompt + new, False, None, temp, top_p, None, 0,
+                                   include_logprobs=True, prompt_lengths=np.full(batch, start))
+    # cache fill over the known tokens (outside the timed region), in multi-token passes
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     if args.sync_steps:
-      run(st, prompt - 1, False)
+      run(st, start - 1, False)
     else:
-      sampler.walk(st, prompt - 1)
+      sampler.walk(st, start - 1)
     torch.cuda.synchronize()
     walk_ms.append((time.perf_counter() - t0) * 1e3)
     return st
@@ -223,10 +257,10 @@ def main():
   run(st, args.steps)
   torch.cuda.synchronize()
   dt = time.perf_counter() - t0
-  toks = st['token_buffer'][:, prompt:prompt + args.warmup + args.steps]
-  assert int(st['step'].item()) == prompt - 1 + args.warmup + args.steps
+  toks = st['token_buffer'][:, start:start + args.warmup + args.steps]
+  assert int(st['step'].item()) == start - 1 + args.warmup + args.steps
   assert bool(((toks >= 0) & (toks < cfg.vocab_size)).all().item())
-  lps = st['logprobs'][:, prompt:prompt + args.warmup + args.steps]
+  lps = st['logprobs'][:, start:start + args.warmup + args.steps]
   assert bool(torch.isfinite(lps).all().item()) and bool((lps <= 0).all().item())
 
   result = {
@@ -240,20 +274,21 @@ def main():
       'higher_is_better': True,
       'scaling': 'weak',
       'vs_baseline': None,
-      'prompt_walk_ms': walk_ms[0],
+      'cache_fill_ms': walk_ms[0],
       'dtype': 'bf16 activations / int4 weights / f32 accumulate',
       'data': 'synthetic (random-init weights, uniform-random prompt ids)',
       'config': {
           'workload': args.workload,
           'shape': name, 'sequences': batch, 'prompt_len': prompt, 'new_tokens': new,
           'quant': f'int4 group {group}', 'lora_rank': rank, 'temperature': temp, 'top_p': top_p,
-          'context_range': [prompt - 1 + args.warmup, prompt - 1 + args.warmup + args.steps],
+          'context_range': [start - 1 + args.warmup, start - 1 + args.warmup + args.steps],
+          'cache_filled_to': start,
       },
   }
 
   # Whole-step algorithmic bytes at the mean context of the timed region.
   wbytes, hbytes = model.weight_bytes(batch)
-  s_mean = prompt + args.warmup + args.steps / 2.0
+  s_mean = start + args.warmup + args.steps / 2.0
   kv_per_tok = cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * 2 * 2
   step_bytes = wbytes + hbytes + batch * s_mean * kv_per_tok
   result['step_hbm'] = {'algorithmic_bytes': step_bytes,
@@ -261,7 +296,8 @@ def main():
                         'frac_of_8TBps': step_bytes / (dt / args.steps) / 8e12}
 
   if not args.no_profile:
-    # Replay the same rollout with HIP events around every launch, sampling every 8th step.
+    # Replay the same rollout with HIP events around every launch: every 8th step of a long run,
+    # every step of a short one.
     lib = _lib.lib()
     st = fresh_state()
     sampler.run_steps(st, args.warmup, sample=True)
@@ -271,13 +307,14 @@ def main():
     tot_cnt = np.zeros_like(cnt)
     ctx_sum, ctx_n = 0.0, 0
     done_steps = 0
+    stride = 8 if args.steps >= 128 else 1
     while done_steps < args.steps:
-      skip = min(7, args.steps - done_steps)
+      skip = min(stride - 1, args.steps - done_steps)
       sampler.run_steps(st, skip, sample=True)
       done_steps += skip
       if done_steps >= args.steps:
         break
-      ctx_sum += prompt + args.warmup + done_steps
+      ctx_sum += start + args.warmup + done_steps
       ctx_n += 1
       cs = sampler._c_state(st)
       rc = lib.tmx_decode_steps_profiled(ctypes.byref(model.desc()), ctypes.byref(cs), _lib.stream(), 1, 1,
@@ -385,7 +422,7 @@ def main():
     # Cache fill (outside the headline metric): the prompt walk above, and the projection kernel that
     # carries it (256-row blocks, MFMA-bound) timed alone on the gate|up shape at the rows of one pass.
     lib = _lib.lib()
-    rows = min(sampler._fill_rows() // batch, 128, prompt - 1) * batch
+    rows = min(sampler._fill_rows() // batch, 128, start - 1) * batch
     pl = model.layers[0]['gate_up']
     xs = torch.randn(rows, pl.k, device='cuda').to(torch.bfloat16)
     ns = lib.tmx_qlora_linear_num_splits(rows, pl.k, pl.n)
@@ -407,7 +444,8 @@ def main():
     g_ms = e0.elapsed_time(e1) / 8
     flops = 2.0 * rows * pl.k * pl.n
     result['prefill'] = {
-        'prompt_tokens_per_s': batch * (prompt - 1) / (walk_ms[0] * 1e-3), 'walk_ms': walk_ms[0],
+        'prompt_tokens_per_s': batch * (start - 1) / (walk_ms[0] * 1e-3), 'walk_ms': walk_ms[0],
+        'walked_tokens_per_sequence': start - 1,
         'rows_per_pass': rows,
         'roofline': {'bound': 'mfma', 'kernel': 'tmx::qlinear_mfma_wide_kernel',
                      'shape': f'{rows} x {pl.k} x {pl.n} (gate|up)', 'avg_launch_ms': g_ms,

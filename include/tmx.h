@@ -300,7 +300,13 @@ typedef struct {
 
 size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int cache_size);
 
-/* Enqueues n_steps iterations of the Sampler's decode loop body
+/* Contract on the step counter: the caller keeps *step + n_steps * max(tokens_per_pass, 1) < buf_len
+ * (<= cache_size).  The library cannot read the device counter on the host; kernels clamp the
+ * column they read and skip writes past buf_len, and token ids are clamped to [0, vocab_size) in
+ * the embedding gather (the reference's JAX gathers clamp too), so a violation yields undefined
+ * tokens but no access outside the buffers.
+ *
+ * Enqueues n_steps iterations of the Sampler's decode loop body
  * (tunix/generate/sampler.py:749-793): read token_buffer[:, *step], run the model with
  * the KV cache, select the next token into column *step + 1, ++*step.  With sample == 0
  * the head and token selection are skipped (cache fill: used to walk over prompt tokens).

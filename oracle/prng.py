@@ -44,9 +44,10 @@ def threefry2x32(k0, k1, c0, c1):
 
 
 def prng_key(seed):
-  """jax.random.PRNGKey(int) -> (hi32, lo32)."""
-  seed = int(seed) & 0xFFFFFFFFFFFFFFFF
-  return np.uint32(seed >> 32), np.uint32(seed & 0xFFFFFFFF)
+  """jax.random.PRNGKey(int) -> (hi32, lo32) with 64-bit types disabled, the reference's
+  configuration: the seed becomes an int32 array (low 32 bits, two's complement), whose logical
+  shift by 32 is 0, so the high key word is 0 for every int, negative ones included."""
+  return np.uint32(0), np.uint32(int(seed) & 0xFFFFFFFF)
 
 
 def fold_in(key, data):

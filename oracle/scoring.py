@@ -7,6 +7,7 @@ packing and without chunking) with process_ids (:257-330) and selective_log_soft
 import numpy as np
 
 from oracle import masks
+from oracle.bf16 import bf16_round
 
 
 def per_token_logps(model, prompt_tokens, completion_tokens, pad_id, temperature=1.0):
@@ -22,7 +23,8 @@ def per_token_logps(model, prompt_tokens, completion_tokens, pad_id, temperature
   keep = comp.shape[1]
   logits = logits[:, -keep - 1:-1, :]                         # :590
   if temperature not in (0.0, 1.0):
-    logits = logits / np.float32(temperature)                 # :591-592
+    # :591-592 `logits /= temperature` on the model's bf16 logits: the quotient is a bf16 array
+    logits = bf16_round(logits / np.float32(temperature))
   return selective_log_softmax(logits, ids[:, -keep:])
 
 

@@ -92,6 +92,8 @@ def oracle_weights(cfg, st, group, lora_alpha, lora_rank, quantized=True):
           'v': lin(f'{p}.attn', 'v_proj', 'w'), 'o': lin(f'{p}.attn', 'o_proj', 'w')}
     if cfg.num_experts:
       def elin(w2):
+        if not quantized:
+          return OL.Linear(w=w2)
         q, s = int4.quantize(w2, group)
         return OL.Linear(q=q, scale=s, group=group)
       lw['router'] = st[f'{p}.mlp.router.kernel']

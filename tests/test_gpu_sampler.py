@@ -515,3 +515,49 @@ def test_packed_checkpoint_round_trip_gives_the_same_rollout(tmp_path):
   b = _sampler(again, cfg, 32)(**kw)
   for x, y, lx, ly in zip(a.tokens, b.tokens, a.logprobs, b.logprobs):
     assert (x == y).all() and np.array_equal(np.asarray(lx), np.asarray(ly))
+
+
+@pytest.mark.parametrize('family', ['llama3', 'qwen3'])
+def test_hf_checkpoint_loader_to_gpu_logits_match_oracle(tmp_path, family):
+  """models/safetensors_loader.py:474 load_and_create_model's path: a Hugging Face checkpoint on disk
+  (transformers random init -> save_pretrained, safetensors) -> checkpoint.model_from_hf (renaming rules
+  of models/llama3/params.py:23-80 / models/qwen3/params.py:47-121 + int4 quantisation) -> decode-step
+  logits on the GPU, against the oracle built from the state the renaming rules give (2e-2)."""
+  transformers = pytest.importorskip('transformers')
+  from tunix_amd import checkpoint as CK
+  torch.manual_seed(3)
+  common = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                num_key_value_heads=2, head_dim=64, max_position_embeddings=64, attention_bias=False,
+                tie_word_embeddings=False)
+  if family == 'llama3':
+    hf = transformers.LlamaForCausalLM(transformers.LlamaConfig(rms_norm_eps=1e-5, mlp_bias=False, **common))
+    cfg = OM.Config('llama3', 2, 512, 256, 512, 4, 64, 2, norm_eps=1e-5)
+  else:
+    hf = transformers.Qwen3ForCausalLM(transformers.Qwen3Config(rms_norm_eps=1e-6, rope_theta=1_000_000.0, **common))
+    cfg = OM.Config('qwen3', 2, 512, 256, 512, 4, 64, 2, rope_theta=1_000_000, norm_eps=1e-6)
+  with torch.no_grad():
+    for name, prm in hf.named_parameters():
+      if 'norm' in name:
+        prm.add_(0.1 * torch.randn_like(prm))
+  hf.to(torch.bfloat16).save_pretrained(str(tmp_path), safe_serialization=True)
+  pcfg = C.product_config(cfg)
+  model = CK.model_from_hf(str(tmp_path), pcfg, group=64)
+  # the oracle takes the renamed state as numpy and quantises it with its own restatement
+  renamed = {k: v.float().numpy() for k, v in CK.load_hf_safetensors(str(tmp_path), pcfg).items()}
+  assert renamed['layers.0.attn.q_proj.w'].shape == (256, 4, 64) and renamed['layers.1.attn.o_proj.w'].shape == (4, 64, 256)
+  oracle = OM.Decoder(cfg, C.oracle_weights(cfg, renamed, 64, 0.0, 0))
+  rng = np.random.default_rng(4)
+  prompts = [rng.integers(3, cfg.vocab_size, 12) for _ in range(3)]
+  ref = OSAM.generate(oracle, cfg, prompts, 6, 32, eos_ids=(-1,), keep_logits=True, max_prompt_length=12)
+  s = _sampler(model, cfg, 32)
+  s.eos_ids = np.array([-1])
+  st = s.init_sample_state(ref['padded_prompt_tokens'], 18, True, None, 0.0, None, None, 0, include_logprobs=True,
+                           prompt_lengths=ref['prompt_lengths'])
+  s.walk(st, 11)
+  for step in range(6):
+    s.run_steps(st, 1, sample=True)
+    got, want = st['logits'].cpu().numpy(), ref['state'].step_logits[step]
+    assert np.abs(got - want).max() <= LOGIT_TOL, (family, step, np.abs(got - want).max())
+    assert np.abs(want).max() > 0.1  # the comparison is not between two all-zero tensors
+    tok = ref['state'].token_buffer[:, 12 + step]
+    st['token_buffer'][:, 12 + step] = torch.from_numpy(tok).to(st['token_buffer'].device)  # teacher forcing

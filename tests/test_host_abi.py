@@ -149,3 +149,106 @@ def test_bench_refuses_more_than_one_gpu():
   import subprocess, sys
   r = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--gpus', '2'], capture_output=True, text=True)
   assert r.returncode != 0 and 'ONE GPU' in r.stderr
+
+
+class _Var:
+  """Stand-in for an nnx.LoRAParam leaf: the array sits in `.value`."""
+
+  def __init__(self, value):
+    self.value = value
+
+
+class _PathKey:
+  """Stand-in for a jax tree path entry (DictKey): the name sits in `.key`."""
+
+  def __init__(self, key):
+    self.key = key
+
+
+def test_flatten_state_takes_what_the_weight_sync_hands_over():
+  import torch
+  from tunix_amd import utils
+  a = np.arange(6, dtype=np.float32).reshape(2, 3)
+  b = np.ones((3, 4), np.float32)
+  want = {'layers.0.attn.q_proj.w_lora_a', 'layers.0.attn.q_proj.w_lora_b'}
+  nested = {'layers': {0: {'attn': {'q_proj': {'w_lora_a': _Var(a), 'w_lora_b': _Var(b)}}}}}
+  by_tuple = {('layers', 0, 'attn', 'q_proj', 'w_lora_a'): a, ('layers', 0, 'attn', 'q_proj', 'w_lora_b'): torch.from_numpy(b)}
+  by_pathkeys = {tuple(_PathKey(k) for k in ('layers', 0, 'attn', 'q_proj', 'w_lora_a')): a,
+                 tuple(_PathKey(k) for k in ('layers', 0, 'attn', 'q_proj', 'w_lora_b')): b}
+  dotted = {'layers.0.attn.q_proj.w_lora_a': a, 'layers.0.attn.q_proj.w_lora_b': b}
+  pure = {'layers': {'0': {'attn': {'q_proj': {'w_lora_a': {'value': a}, 'w_lora_b': {'value': b}}}}}}
+  as_list = {'layers': [{'attn': {'q_proj': {'w_lora_a': a, 'w_lora_b': b}}}]}
+  for tree in (nested, by_tuple, by_pathkeys, dotted, pure, as_list):
+    flat = utils.flatten_state(tree)
+    assert set(flat) == want
+    np.testing.assert_array_equal(flat['layers.0.attn.q_proj.w_lora_a'].float().numpy(), a)
+    assert tuple(flat['layers.0.attn.q_proj.w_lora_b'].shape) == (3, 4)
+
+
+class _LoraStub:
+  """Model stand-in for the weight-sync logic: LoRA state in, LoRA state out, with the product's checks."""
+
+  def __init__(self):
+    import torch
+    self.config = ModelConfig.toy()
+    self.device = 'cpu'
+    self.state = {'layers.0.attn.q_proj.w_lora_a': torch.zeros(256, 8, dtype=torch.bfloat16),
+                  'layers.0.attn.q_proj.w_lora_b': torch.zeros(8, 256, dtype=torch.bfloat16)}
+
+  def lora_state(self):
+    return dict(self.state)
+
+  def update_lora(self, state):
+    import torch
+    from tunix_amd.model import QLoRAModel
+    QLoRAModel.check_lora_state(self.state, state)
+    self.state = {k: torch.as_tensor(v).to(torch.bfloat16).reshape(self.state[k].shape) for k, v in state.items()}
+
+
+def test_update_params_accepts_nested_states_and_keeps_the_reference_errors():
+  from tunix_amd.sampler import Sampler
+  c = ModelConfig.toy()
+  s = Sampler(_LoraStub(), C.ToyTokenizer(), CacheConfig(8, c.num_layers, c.num_kv_heads, c.head_dim))
+  a = np.full((256, 8), 0.5, np.float32)
+  # q_proj B arrives as the reference's [r, N, H] Einsum shape
+  b = np.full((8, 4, 64), 0.25, np.float32)
+  s.update_params({'layers': {0: {'attn': {'q_proj': {'w_lora_a': _Var(a), 'w_lora_b': _Var(b)}}}}})
+  got = s.transformer_state
+  assert got['layers.0.attn.q_proj.w_lora_a'].dtype.is_floating_point
+  assert float(got['layers.0.attn.q_proj.w_lora_a'].float().mean()) == 0.5
+  assert float(got['layers.0.attn.q_proj.w_lora_b'].float().mean()) == 0.25
+  # partial update: only A
+  s.update_params({('layers', 0, 'attn', 'q_proj', 'w_lora_a'): a * 2})
+  assert float(s.transformer_state['layers.0.attn.q_proj.w_lora_a'].float().mean()) == 1.0
+  with pytest.raises(ValueError, match='same structure'):
+    s.update_params({'layers': {0: {'attn': {'z_proj': {'w_lora_a': a}}}}})
+  with pytest.raises(ValueError, match='same shape'):
+    s.update_params({'layers.0.attn.q_proj.w_lora_a': np.zeros((256, 4), np.float32)})
+  with pytest.raises(ValueError, match='same structure'):
+    s.transformer_state = {'layers.0.attn.q_proj.w_lora_a': a}  # the setter wants the whole LoRA state
+
+
+def test_seed_words_follow_prngkey_without_x64():
+  from oracle import prng
+  from tunix_amd.sampler import _seed_key
+  for seed in (0, 42, -1, 2 ** 32 + 5, 2 ** 40):
+    assert _seed_key(seed) == (0, seed & 0xFFFFFFFF)
+    assert tuple(int(w) for w in prng.prng_key(seed)) == (0, seed & 0xFFFFFFFF)
+  assert _seed_key(None) == (0, 0)
+  assert _seed_key(np.array([7, 9], np.uint32)) == (7, 9)
+  typed = type('K', (), {'_base_array': np.array([1, 2], np.uint32)})()
+  assert _seed_key(typed) == (1, 2)
+  with pytest.raises(ValueError):
+    _seed_key(np.arange(3))
+
+
+def test_token_ids_outside_the_vocabulary_are_rejected_before_the_gpu():
+  s = _sampler(cache_size=16)
+  v = ModelConfig.toy().vocab_size
+  for bad in ([[3, v]], [[-2, 4]]):
+    with pytest.raises(ValueError, match='outside the vocabulary'):
+      s(prompt_token_ids=bad, max_generation_steps=2)
+  with pytest.raises(ValueError, match='outside the vocabulary'):
+    s.per_token_logps(np.array([[3, 4]]), np.array([[5, v + 7]]))
+  with pytest.raises(NotImplementedError, match='echo'):
+    s(prompt_token_ids=[[3, 4]], max_generation_steps=2, echo=True, return_logits=True)

@@ -338,6 +338,70 @@ def test_dense_forward_matches_transformers(family):
     np.testing.assert_allclose(lg[:, 0], want[:, step], atol=1e-3)
 
 
+def test_moe_forward_matches_transformers():
+  """The routed-expert layer (tunix/models/qwen3/model.py:894-939: f32 softmax over all experts,
+  top-k, weights renormalised over the top-k, sum of weighted expert SwiGLU outputs) against
+  transformers' Qwen3MoeForCausalLM with norm_topk_prob=True, random weights, fp32."""
+  import torch
+  transformers = pytest.importorskip('transformers')
+  torch.manual_seed(1)
+  e, topk, f = 8, 2, 32
+  hf_cfg = transformers.Qwen3MoeConfig(
+      vocab_size=128, hidden_size=64, intermediate_size=96, moe_intermediate_size=f, num_hidden_layers=2,
+      num_attention_heads=4, num_key_value_heads=2, head_dim=16, max_position_embeddings=64, attention_bias=False,
+      tie_word_embeddings=False, num_experts=e, num_experts_per_tok=topk, norm_topk_prob=True, decoder_sparse_step=1,
+      mlp_only_layers=[], rms_norm_eps=1e-6, rope_theta=10_000.0)
+  hf = transformers.Qwen3MoeForCausalLM(hf_cfg).float().eval()
+  with torch.no_grad():
+    for name, prm in hf.named_parameters():
+      if 'norm' in name:
+        prm.add_(0.1 * torch.randn_like(prm))
+      if name.endswith('mlp.gate.weight'):
+        prm.mul_(20.0)  # spread-out routing scores: top-k choices far from ties
+      if 'experts' in name:
+        prm.mul_(5.0)   # expert outputs large enough that a wrong routing weight or expert shows at 1e-3
+  sd = hf.state_dict()
+  cfg = OM.Config('qwen3', 2, 128, 64, f, 4, 16, 2, rope_theta=10_000, norm_eps=1e-6, num_experts=e, experts_per_tok=topk)
+  g = lambda k: sd[k].detach().numpy().astype(np.float32)
+  d, n, kh, h = cfg.embed_dim, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+  st = {'embedder.input_embedding': g('model.embed_tokens.weight'), 'final_norm.w': g('model.norm.weight'),
+        'lm_head.w': g('lm_head.weight').T.copy()}
+  for i in range(cfg.num_layers):
+    p, hp = f'layers.{i}', f'model.layers.{i}'
+    st[f'{p}.input_layernorm.w'] = g(f'{hp}.input_layernorm.weight')
+    st[f'{p}.post_attention_layernorm.w'] = g(f'{hp}.post_attention_layernorm.weight')
+    st[f'{p}.attn.q_proj.w'] = g(f'{hp}.self_attn.q_proj.weight').T.reshape(d, n, h)
+    st[f'{p}.attn.k_proj.w'] = g(f'{hp}.self_attn.k_proj.weight').T.reshape(d, kh, h)
+    st[f'{p}.attn.v_proj.w'] = g(f'{hp}.self_attn.v_proj.weight').T.reshape(d, kh, h)
+    st[f'{p}.attn.o_proj.w'] = g(f'{hp}.self_attn.o_proj.weight').T.reshape(n, h, d)
+    st[f'{p}.attn.q_norm.w'] = g(f'{hp}.self_attn.q_norm.weight')
+    st[f'{p}.attn.k_norm.w'] = g(f'{hp}.self_attn.k_norm.weight')
+    st[f'{p}.mlp.router.kernel'] = g(f'{hp}.mlp.gate.weight').T.copy()                # [D, E]
+    gu = g(f'{hp}.mlp.experts.gate_up_proj')                                           # [E, 2F, D]: gate rows, then up rows
+    st[f'{p}.mlp.gate_proj'] = np.ascontiguousarray(gu[:, :f, :].transpose(0, 2, 1))  # [E, D, F]
+    st[f'{p}.mlp.up_proj'] = np.ascontiguousarray(gu[:, f:, :].transpose(0, 2, 1))
+    st[f'{p}.mlp.down_proj'] = np.ascontiguousarray(g(f'{hp}.mlp.experts.down_proj').transpose(0, 2, 1))  # [E, F, D]
+  dec = OM.Decoder(cfg, C.oracle_weights(cfg, st, 64, 0.0, 0, quantized=False), F32)
+  toks = torch.randint(0, 128, (2, 9))
+  with torch.no_grad():
+    out = hf(toks, output_router_logits=True)
+  want = out.logits.numpy()
+  pos = np.tile(np.arange(9), (2, 1))
+  got, _ = dec(toks.numpy(), pos, None, OMK.make_causal_attn_mask(np.ones((2, 9), bool), 9))
+  np.testing.assert_allclose(got, want, atol=1e-3)
+  # the routing itself: the same experts per token as the library's top-k of its router logits
+  for i, rl in enumerate(out.router_logits):
+    hf_idx = np.sort(torch.topk(torch.softmax(rl.float(), -1), topk, dim=-1).indices.numpy(), axis=-1)
+    np.testing.assert_array_equal(np.sort(np.asarray(dec.routed[i]).reshape(-1, topk), axis=-1), hf_idx)
+  # a wrong renormalisation would show: without it the logits move by far more than the tolerance
+  hf.config.norm_topk_prob = False
+  for layer in hf.model.layers:
+    layer.mlp.gate.norm_topk_prob = False
+  with torch.no_grad():
+    other = hf(toks).logits.numpy()
+  assert np.abs(other - want).max() > 1e-2
+
+
 def test_oracle_sampler_loop_invariants():
   cfg = OM.Config('llama3', 1, 64, 64, 64, 2, 32, 2)
   st = C.make_state(cfg, 13, 0)

@@ -53,7 +53,8 @@ __global__ __launch_bounds__(AttnWaves<G>::value * 64) void gqa_decode_kernel(At
   const int pg = lane / LPP, dl = lane % LPP;  // lane group, 8-element slice index
   const int tpp = a.tpp > 0 ? a.tpp : 1;
   const int seq = b / tpp;                    // b: query row of this pass
-  const int step = *a.step + b % tpp;
+  // newest valid slot; clamped into the cache and the mask row so that a caller that oversteps reads in bounds
+  const int step = min(*a.step + b % tpp, min(a.C, a.buf_len) - 1);
   // the splits share the VALID positions 0 .. step (not the cache size) in chunks of whole
   // 32 positions, so that every split has work at any context length
   const int chunk = (((step + a.nsplit) / a.nsplit) + 31) & ~31;
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(256) void gqa_fill_kernel(AttnArgs a) {
   const int kvh = blockIdx.x, seq = blockIdx.y, tblk = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int h = lane >> 5, qi = lane & 31;
-  const int T = a.tpp, step0 = *a.step;
+  const int T = a.tpp, step0 = max(min(*a.step, min(a.C, a.buf_len) - T), 0);  // clamped: every slot read lies in the cache
   const int tok = tblk * TQ + wave * TPW + qi / G, g = qi % G;
   const int tok_l = tok < T ? tok : T - 1;
   const int limit = step0 + tok_l;  // newest slot this query sees

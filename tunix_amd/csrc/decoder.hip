@@ -187,6 +187,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     {  // embedding gather + first input norm + this step's RoPE table
       RowNormArgs a = {};
       a.embed = (const uint16_t*)m->embed;
+      a.vocab = m->vocab_size;
       a.token_buffer = s->token_buffer;
       a.step = s->step;
       a.buf_len = L;

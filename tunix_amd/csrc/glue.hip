@@ -178,8 +178,11 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
   const uint16_t* src = nullptr;
   if (a.embed) {
     const int tpp = a.tpp > 0 ? a.tpp : 1;
-    const int seq = m / tpp, step = *a.step + m % tpp;
-    const int tok = a.token_buffer[(size_t)seq * a.buf_len + step];
+    // column and id are clamped into range like the reference's gathers (jnp indexing clamps), so a
+    // caller that oversteps the buffer or feeds an id outside the vocabulary reads a valid row
+    const int seq = m / tpp, step = min(*a.step + m % tpp, a.buf_len - 1);
+    int tok = a.token_buffer[(size_t)seq * a.buf_len + step];
+    if (a.vocab > 0) tok = min(max(tok, 0), a.vocab - 1);
     src = a.embed + (size_t)tok * a.D;
     if (a.rope_tab && (int)threadIdx.x < a.half) {
       const float pos = (float)a.positions[(size_t)seq * a.buf_len + step];
@@ -339,7 +342,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(RopeArgs a) {
   const int head = blockIdx.x, b = blockIdx.y, B = gridDim.y, lane = threadIdx.x;
   const int half = a.H >> 1;
   const int tpp = a.tpp > 0 ? a.tpp : 1;
-  const int seq = b / tpp, step = *a.step + b % tpp;  // b: row of this pass
+  const int seq = b / tpp, step = min(*a.step + b % tpp, a.buf_len - 1);  // b: row of this pass (column clamped into the buffer)
   const bool active = lane < half;
   const int ntot = (a.N + 2 * a.Kh) * a.H;
   const int kind = head < a.N ? 0 : (head < a.N + a.Kh ? 1 : 2);  // q, k, v

@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
     const int tpp = a.tpp > 0 ? a.tpp : 1;
     const int prow = a.row_base + row;  // row of the pass
     target[m] = (score && row < a.M)
-                    ? a.token_buffer[(size_t)(prow / tpp) * a.buf_len + *a.step + prow % tpp + 1] : -1;
+                    ? a.token_buffer[(size_t)(prow / tpp) * a.buf_len + min(*a.step + prow % tpp + 1, a.buf_len - 1)] : -1;
   }
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
         float z = logit, key = logit;
         if (score) {
           // the "best" candidate is the given next token: its z is what the log-prob needs
-          z = score_clip(logit / a.temperature);
+          z = score_clip(rbf(logit / a.temperature));  // bf16 logits divided in place stay bf16 (rl/common.py:591-592)
           key = (v == target[m]) ? 0.f : -INFINITY;
         } else if (a.mode == TMX_SAMPLE_TOP_P) {
           z = logit / a.temperature;
@@ -260,11 +260,13 @@ __global__ __launch_bounds__(256) void head_finalize_kernel(HeadArgs a) {
       const int tpp = a.tpp > 0 ? a.tpp : 1;
       const int prow = a.row_base + row;
       // selective_log_softmax: logit - logsumexp, with logsumexp = max + log(sum exp(z - max))
-      if (a.logprobs)
-        a.logprobs[(size_t)(prow / tpp) * a.buf_len + *a.step + prow % tpp + 1] = best.z - (mx + logf(se));
+      const int scol = *a.step + prow % tpp + 1;
+      if (a.logprobs && scol < a.buf_len)
+        a.logprobs[(size_t)(prow / tpp) * a.buf_len + scol] = best.z - (mx + logf(se));
       return;
     }
     const int col = *a.step + 1;
+    if (col >= a.buf_len) return;  // a caller that steps past the buffer gets no write instead of a stray one
     const int tok = best.idx;
     a.token_buffer[(size_t)row * a.buf_len + col] = tok;
     if (a.logprobs) a.logprobs[(size_t)row * a.buf_len + col] = (best.z - mx) - logf(se);
@@ -388,7 +390,7 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
   uint32_t key0 = 0, key1 = 0;
   if (sampling) threefry2x32(a.k0, a.k1, 0u, (uint32_t)*a.step, key0, key1);
   const int tpp = a.tpp > 0 ? a.tpp : 1;
-  const int target = score ? a.token_buffer[(size_t)(tok_l / tpp) * a.buf_len + *a.step + tok_l % tpp + 1] : -1;
+  const int target = score ? a.token_buffer[(size_t)(tok_l / tpp) * a.buf_len + min(*a.step + tok_l % tpp + 1, a.buf_len - 1)] : -1;
   float mx = kNegBig, se = 0.f;
   Best best = {-INFINITY, -INFINITY, 0x7FFFFFFF};
   // (unrolled by construction: a loop the compiler declines to unroll would index the accumulators
@@ -400,7 +402,7 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
       const float logit = rbf(acc[m][r]);
       float z = logit, key = logit;
       if (score) {
-        z = score_clip(logit / a.temperature);
+        z = score_clip(rbf(logit / a.temperature));  // bf16 logits divided in place stay bf16 (rl/common.py:591-592)
         key = (v == target) ? 0.f : -INFINITY;
       } else if (sampling) {
         z = logit / a.temperature;

@@ -131,6 +131,7 @@ __global__ __launch_bounds__(kSelThreads) void nucleus_select_kernel(NucleusArgs
     }
     const int tok = (int)(a.vals[base + best.idx] - (uint32_t)base);
     const int col = *a.step + 1;
+    if (col >= a.buf_len) return;
     a.token_buffer[(size_t)row * a.buf_len + col] = tok;
     if (a.logprobs) a.logprobs[(size_t)row * a.buf_len + col] = (best.z - mx) - logf(se);
     bool hit = false;

@@ -68,6 +68,7 @@ struct LoraIn {
 struct RowNormArgs {
   // source of the row: an embedding gather (embed != null) or y (+ LoRA) (+ residual)
   const uint16_t* embed;        // [V, D]
+  int vocab;                    // V (ids are clamped to [0, V)); 0: no clamp
   const int32_t* token_buffer;  // [B, L]
   const int32_t* step;          // device scalar: column of token_buffer to read
   int buf_len;

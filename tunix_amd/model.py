@@ -278,20 +278,27 @@ class QLoRAModel:
           col += width
     return out
 
-  def update_lora(self, state):
-    """LoRA-only replacement (tunix/generate/sampler.py:340-354): `state` must have
-    exactly the keys and shapes of lora_state(); base int4 weights are untouched."""
-    cur = self.lora_state()
+  @staticmethod
+  def check_lora_state(cur, state):
+    """The reference's checks on a replacement state (tunix/generate/sampler.py:281-332): same
+    paths, same shapes (3-D Einsum shapes are accepted for their flattened 2-D counterparts)."""
     if set(state.keys()) != set(cur.keys()):
       raise ValueError('New state must have the same structure as the old state.'
                        f' {sorted(cur.keys())[:3]}... vs {sorted(state.keys())[:3]}...')
     for k, v in state.items():
       v = torch.as_tensor(v)
-      ok = v.numel() == cur[k].numel() and (
+      ok = v.numel() == cur[k].numel() and v.dim() >= 2 and (
           v.reshape(cur[k].shape[0], -1).shape == cur[k].shape or v.reshape(-1, cur[k].shape[-1]).shape == cur[k].shape)
+      # a flattened axis must be one the Einsum layout really has: first or last dimension kept
+      ok = ok and (v.shape[0] == cur[k].shape[0] or v.shape[-1] == cur[k].shape[-1])
       if not ok:
         raise ValueError('New state must have the same shape, dtype and sharding as the old state.'
                          f' {k}: {tuple(v.shape)} vs {tuple(cur[k].shape)}')
+
+  def update_lora(self, state):
+    """LoRA-only replacement (tunix/generate/sampler.py:340-354): `state` must have
+    exactly the keys and shapes of lora_state(); base int4 weights are untouched."""
+    self.check_lora_state(self.lora_state(), state)
     for i, layer in enumerate(self.layers):
       for key, names, pre, wk in (('qkv', ('q_proj', 'k_proj', 'v_proj'), 'attn', 'w'),
                                   ('o', ('o_proj',), 'attn', 'w'),

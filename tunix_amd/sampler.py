@@ -57,12 +57,19 @@ class TokenizerAdapter:
 
 
 def _seed_key(seed):
-  """jax.random.PRNGKey(int) as (hi32, lo32); a 2-word key passes through."""
+  """The two threefry key words (hi32, lo32) of a seed.  An int goes through
+  jax.random.PRNGKey with 64-bit types disabled, as in the reference (sampler.py:938-941): the
+  high word is 0 and the low word the seed's low 32 bits, negative seeds included.  A raw 2-word
+  key (uint32[2]) passes through; a typed key array is unwrapped to its key data first."""
   if seed is None:
     seed = 0
   if isinstance(seed, (int, np.integer)):
-    seed = int(seed) & 0xFFFFFFFFFFFFFFFF
-    return seed >> 32, seed & 0xFFFFFFFF
+    return 0, int(seed) & 0xFFFFFFFF
+  for attr in ('_base_array', 'key_data'):  # jax typed keys (jax.random.key): the wrapped uint32[2]
+    inner = getattr(seed, attr, None)
+    if inner is not None and not callable(inner):
+      seed = inner
+      break
   arr = np.asarray(seed).astype(np.uint32).reshape(-1)
   if arr.size != 2:
     raise ValueError('seed must be an int or a 2-word key')
@@ -107,13 +114,19 @@ class Sampler:
 
   @transformer_state.setter
   def transformer_state(self, state):
-    self._transformer.update_lora(state)
+    self._transformer.update_lora(utils.flatten_state(state))
 
   def update_params(self, updated_weights, filter_types=None):
-    """LoRA weight sync between rollouts (tunix/rl/rl_cluster.py:1279-1294 passes the
-    LoRA-filtered state).  New tensors are cast to the rollout precision (bf16)."""
+    """LoRA weight sync between rollouts.  RLEngine.sync_weights passes
+    nnx.state(actor, nnx.LoRAParam) (tunix/rl/rl_cluster.py:1279-1294); the reference flattens
+    it with to_flat_dict, casts to the rollout precision and merges it over the old parameters
+    (tunix/generate/sampler.py:361-392).  Accepted here: a flat mapping under dotted names, a
+    mapping keyed by path tuples, or a nested mapping / state object (anything with .items()),
+    with array leaves or variable-like leaves that carry the array in `.value`.  Tensors are
+    cast to bf16; a path the model does not have, or a tensor of another shape, raises the
+    reference's "same structure" / "same shape" errors."""
     del filter_types
-    flat = {k: torch.as_tensor(v) for k, v in dict(updated_weights).items()}
+    flat = utils.flatten_state(updated_weights)
     merged = dict(self._transformer.lora_state())
     unknown = set(flat) - set(merged)
     if unknown:
@@ -148,6 +161,15 @@ class Sampler:
     ids = np.asarray(all_input_ids, dtype=np.int32)
     b, p = ids.shape
     pad = self.tokenizer.pad_id()
+    # Every column of the buffer is gathered from the embedding table at some step (pad columns
+    # included), so every id must be a valid row.  The reference's JAX gather clamps silently.
+    vocab = self._transformer.config.vocab_size
+    if ids.size and (ids.min() < 0 or ids.max() >= vocab):
+      bad = ids[(ids < 0) | (ids >= vocab)]
+      raise ValueError(f'token id {int(bad[0])} is outside the vocabulary [0, {vocab}) '
+                       '(prompt ids and the tokenizer\'s pad_id must be valid embedding rows)')
+    if not 0 <= pad < vocab:
+      raise ValueError(f'pad_id {pad} is outside the vocabulary [0, {vocab})')
     token_buffer = np.full((b, total_sampling_steps), pad, dtype=np.int32)
     token_buffer[:, :p] = ids
     input_mask = np.ones((b, total_sampling_steps), dtype=bool)
@@ -320,6 +342,11 @@ class Sampler:
                prompt_token_ids=None):
     if images is not None or audios is not None:
       raise NotImplementedError('image / audio inputs are outside this decode path')
+    if return_logits and echo:
+      # the reference slices its logits buffer from the first prompt token on (sampler.py:1045-1052);
+      # the cache fill here computes no prompt logits, so only generated-step logits exist
+      raise NotImplementedError('return_logits with echo=True needs prompt-position logits, which the cache fill '
+                                'does not compute; call with echo=False')
     self.eos_ids = np.array(list(eos_tokens) if eos_tokens else [self.tokenizer.eos_id()])
     exact_input = prompt_token_ids is not None
     tokens = utils.resolve_prompt_tokens(

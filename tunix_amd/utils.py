@@ -104,37 +104,101 @@ def as_token_ids(value):
   return array
 
 
+def _token_rows(prompt_token_ids, budget, max_length_name, single_output_per_row):
+  """Validated int32 rows of caller-supplied token ids (error texts as the reference's)."""
+  if len(prompt_token_ids) == 0:
+    raise ValueError('prompt_token_ids must not be empty')
+  if not single_output_per_row:
+    raise ValueError('prompt_token_ids requires exactly one output per row')
+  rows = [as_token_ids(r) for r in prompt_token_ids]
+  if budget is not None and max((len(r) for r in rows), default=0) > budget:
+    raise ValueError(f'prompt plus max_generation_steps exceeds {max_length_name}')
+  return rows
+
+
 def resolve_prompt_tokens(input_strings, prompt_token_ids, tokenize_fn, *, max_generation_steps=0,
                           max_total_length=None, max_length_name='max_model_len',
                           single_output_per_row=True):
-  if (input_strings is None) == (prompt_token_ids is None):
+  """One int32 id row per prompt, from text (tokenised here) or from ids given as they are."""
+  have_text, have_ids = input_strings is not None, prompt_token_ids is not None
+  if have_text == have_ids:
     raise ValueError('Provide exactly one of input_strings or prompt_token_ids')
-  if prompt_token_ids is not None:
-    if len(prompt_token_ids) == 0:
-      raise ValueError('prompt_token_ids must not be empty')
-    if not single_output_per_row:
-      raise ValueError('prompt_token_ids requires exactly one output per row')
-    rows = [as_token_ids(r) for r in prompt_token_ids]
-    if max_total_length is not None and any(
-        len(r) + max_generation_steps > max_total_length for r in rows):
-      raise ValueError(f'prompt plus max_generation_steps exceeds {max_length_name}')
-    return rows
-  if isinstance(input_strings, np.ndarray):
-    input_strings = input_strings.tolist()
-  if isinstance(input_strings, str):
-    input_strings = [input_strings]
-  if len(input_strings) == 0:
+  if have_ids:
+    budget = None if max_total_length is None else max_total_length - max_generation_steps
+    return _token_rows(prompt_token_ids, budget, max_length_name, single_output_per_row)
+  texts = input_strings.tolist() if isinstance(input_strings, np.ndarray) else input_strings
+  texts = [texts] if isinstance(texts, str) else texts
+  if len(texts) == 0:
     raise ValueError('input_strings must not be empty')
-  return [np.asarray(tokenize_fn(str(s)), dtype=np.int32) for s in input_strings]
+  return [np.asarray(tokenize_fn(str(t)), dtype=np.int32) for t in texts]
 
 
 def left_pad_prompt_tokens(prompt_ids, max_prompt_length, pad_value, *, max_allowed_length=None):
-  prompt_lengths = np.array([len(x) for x in prompt_ids], dtype=np.int32)
-  longest = int(prompt_lengths.max())
-  if max_prompt_length is None or max_prompt_length < longest:
-    max_prompt_length = next_power_of_2(longest)
-    if max_allowed_length is not None and longest <= max_allowed_length:
-      max_prompt_length = min(max_prompt_length, max_allowed_length)
-  rows = [pad_to_length(np.asarray(x, dtype=np.int32), max_prompt_length, pad_value, left=True)
-          for x in prompt_ids]
-  return np.array(rows, dtype=np.int32), prompt_lengths, max_prompt_length
+  """(left-padded int32 [B, P], true lengths, P).  P is the caller's max_prompt_length when every
+  prompt fits it; otherwise the longest prompt rounded up to a power of two (one compiled shape
+  per bucket in the reference), capped by max_allowed_length when the longest prompt still fits."""
+  lengths = np.fromiter((len(r) for r in prompt_ids), dtype=np.int32, count=len(prompt_ids))
+  longest = int(lengths.max())
+  width = max_prompt_length
+  if width is None or width < longest:
+    width = next_power_of_2(longest)
+    if max_allowed_length is not None and longest <= max_allowed_length < width:
+      width = max_allowed_length
+  padded = np.full((len(prompt_ids), width), pad_value, dtype=np.int32)
+  for i, r in enumerate(prompt_ids):
+    if len(r):
+      padded[i, width - len(r):] = np.asarray(r, dtype=np.int32)
+  return padded, lengths, width
+
+
+def _leaf_array(leaf):
+  """Array held by a state leaf: variable-like objects (nnx.Param / nnx.LoRAParam) carry it in
+  `.value` (newer releases: `get_value()`); bf16 arrays of array libraries without a native
+  numpy dtype are taken over by their bit pattern."""
+  import torch
+  for _ in range(2):
+    if isinstance(leaf, (torch.Tensor, np.ndarray)):
+      break
+    if hasattr(leaf, 'value'):
+      leaf = leaf.value
+    elif hasattr(leaf, 'get_value'):
+      leaf = leaf.get_value()
+  if isinstance(leaf, torch.Tensor):
+    return leaf
+  arr = np.asarray(leaf)
+  if arr.dtype.kind == 'V' or arr.dtype.name == 'bfloat16':
+    if arr.dtype.itemsize != 2:
+      raise ValueError(f'unsupported parameter dtype {arr.dtype}')
+    return torch.from_numpy(np.ascontiguousarray(arr).view(np.int16).copy()).view(torch.bfloat16)
+  return torch.from_numpy(np.ascontiguousarray(arr))
+
+
+def flatten_state(tree):
+  """Flat {dotted path: tensor} of a parameter tree, the counterpart of the reference's
+  to_flat_dict (tunix/rl/utils.py:72-78, keys = tuples of path parts) for what the weight sync
+  hands over: nested mappings or state objects (anything with .items()), mappings keyed by
+  path tuples, lists / tuples (index as path part), leaves that are arrays or variable-like
+  objects with the array in `.value`.  Integer path parts (layer indices) print as digits."""
+  out = {}
+
+  def is_node(x):
+    return hasattr(x, 'items') and callable(x.items) and not hasattr(x, 'shape')
+
+  def walk(prefix, node):
+    if is_node(node):
+      for k, v in node.items():
+        parts = tuple(k) if isinstance(k, tuple) else (k,)
+        walk(prefix + tuple(str(getattr(p, 'key', p)) for p in parts), v)
+    elif isinstance(node, (list, tuple)) and not (node and isinstance(node[0], (int, float, np.number))):
+      for i, v in enumerate(node):
+        walk(prefix + (str(i),), v)
+    else:
+      name = '.'.join(prefix)
+      if name.endswith('.value'):  # pure-dict dumps of variable objects
+        name = name[:-len('.value')]
+      if name in out:
+        raise ValueError(f'duplicate parameter path {name!r}')
+      out[name] = _leaf_array(node)
+
+  walk((), tree)
+  return out
