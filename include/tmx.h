@@ -198,9 +198,11 @@ int tmx_head_sample(void* stream, const void* x, const void* head_w, int M, int 
  * order, ties in index order; probs = softmax over the candidates; a candidate is dropped when
  * the cumulative probability before it exceeds top_p; token = Gumbel-max over the survivors
  * with the noise of rank i of row m drawn at linear index m * k + i; logprob =
- * log_softmax(z)[token] over the full vocabulary.  Same outputs as tmx_head_sample.
- * nucleus_workspace: tmx_nucleus_workspace_bytes(M, V) bytes (sort keys, sorted pairs and the
- * radix sort's scratch; the size is asked of the sort routine and is 0 without a device). */
+ * log_softmax(z)[token] over the full vocabulary.  Same outputs as tmx_head_sample.  Nothing is
+ * sorted: the logits are bf16, so ranks and cumulative probabilities follow from per-row counts
+ * of the 65 536 possible values (three launches after the head kernel, no library call).
+ * nucleus_workspace: tmx_nucleus_workspace_bytes(M, V) bytes (one 16-bit key per logit, the
+ * per-row value tables and the slice winners); 0 for an unsupported shape. */
 size_t tmx_nucleus_workspace_bytes(int M, int V);
 int tmx_head_sample_nucleus(void* stream, const void* x, const void* head_w, int M, int D, int V,
                             float temperature, float top_p, int top_k, uint32_t seed_hi,
@@ -318,7 +320,7 @@ int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state,
  * (fewer host launches; what the reference gets from jit-compiling the while_loop).  Unlike
  * tmx_decode_steps this call WAITS for its replays before it returns (the graph is private
  * to the call), creates and destroys a stream, an event and a graph, and falls back to plain
- * launches for the sorting branch of top-p, for n_steps < 4 or when capture is unavailable. */
+ * launches for n_steps < 4 or when capture is unavailable. */
 int tmx_decode_steps_graph(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
                            int n_steps, int sample);
 

@@ -422,9 +422,6 @@ extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state*
 extern "C" int tmx_decode_steps_graph(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
                                       int n_steps, int sample) {
   if (n_steps < 4 || !m || !s) return decode_steps_impl(m, s, stream, n_steps, sample, nullptr);
-  // the sorting branch of top-p calls a library sort that records memset nodes: keep it eager
-  if (sample && s->sampling_mode == TMX_SAMPLE_TOP_P && (s->top_p < 1.0f || s->top_k > 0))
-    return decode_steps_impl(m, s, stream, n_steps, sample, nullptr);
   int rc = decode_steps_impl(m, s, stream, 1, sample, nullptr);
   if (rc != TMX_OK) return rc;
   hipStream_t user = (hipStream_t)stream;

@@ -151,6 +151,7 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
     float mx = kNegBig, se = 0.f;
     Best best = {-INFINITY, -INFINITY, 0x7FFFFFFF};
     if (live && row < a.M) {
+      uint64_t packed = 0;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int v = v0 + acc_row(r, lane);
@@ -166,12 +167,15 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void head_kernel(HeadArgs a) 
         } else if (a.mode == TMX_SAMPLE_TOP_P) {
           z = logit / a.temperature;
           if (a.sort_keys) {
-            // ascending key order = descending logit = descending z (T > 0; -0 == +0), rows kept
-            // apart by the high word.  The logit is a bf16 value, so the low 16 key bits only
-            // repeat the sign and the sort leaves them out.
-            const uint32_t zb = __float_as_uint(logit + 0.0f);
-            const uint32_t ord = (zb & 0x80000000u) ? ~zb : (zb | 0x80000000u);
-            a.sort_keys[(size_t)row * a.V + v] = ((uint64_t)(a.row_off + row) << 32) | (uint32_t)~ord;
+            // 16-bit key whose ascending order is the descending order of the logit (= of z, T > 0;
+            // -0 counts as +0): non-negative values count down from 0x7FFF, negative ones up from 0x8000
+            const uint32_t zb = __float_as_uint(logit + 0.0f) >> 16;
+            // registers 4 q .. 4 q + 3 hold four consecutive vocabulary rows: one 8-byte store
+            packed |= (uint64_t)((zb & 0x8000u) ? zb : (~zb & 0x7FFFu)) << (16 * (r & 3));
+            if ((r & 3) == 3) {
+              *reinterpret_cast<uint64_t*>(a.sort_keys + (size_t)row * a.V + v - 3) = packed;
+              packed = 0;
+            }
             key = z;
           } else {
             uint32_t o0, o1;

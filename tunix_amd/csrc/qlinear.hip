@@ -809,7 +809,6 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   const int KT = a.K >> 6, nsteps = KT / TS, last_step = nsteps - 1;  // host: K % (64 TS) == 0
   const int gs = __builtin_ctz(a.G >> 6), KG = a.K / a.G;
   const int nb = (int)blockIdx.x * 2 + (cw & 1) + (cw >> 1) * a.pair_off;  // host: F % 64 == 0
-  TMX_STAMP(0);
 
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qw, (uint32_t)(a.N >> 5) * KT * 1024u);
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scales, (uint32_t)(a.N >> 5) * KG * 64u);
@@ -933,20 +932,15 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   dma_x(0, 0);
   static_for<TPW>([&](auto jc) __attribute__((always_inline)) { load_w_tile(0, jc); });
   if constexpr (FUSE) load_l(0);
-  TMX_STAMP(1);
   __builtin_amdgcn_sched_barrier(0);
   __builtin_amdgcn_s_waitcnt(0x0F70 | (kYounger & 15) | ((kYounger >> 4) << 14));
   __syncthreads();
-  TMX_STAMP(2);
   const int npairs = nsteps / 2;
   for (int g = 0; g < npairs; ++g) {
     do_step(2 * g, IC<0>{});
-    TMX_STAMP(3 + 2 * g);
     do_step(2 * g + 1, IC<1>{});
-    TMX_STAMP(4 + 2 * g);
   }
   if (nsteps & 1) do_step(nsteps - 1, IC<0>{});
-  TMX_STAMP(29);
 
   // ---- epilogue (the slab is free: the last step ended with a barrier) ----
   // LDS regions (f32 unless noted): P [8 waves][MT][16][64] partial LoRA tiles, later reused as
@@ -1036,7 +1030,6 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
         a.y_bf16[(size_t)row * a.ldy + col] = f2bf(rbf(g * sg) * u);
       }
   }
-  TMX_STAMP(30);
 }
 
 template <int MT, bool FUSE>

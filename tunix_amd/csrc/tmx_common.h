@@ -133,19 +133,6 @@ __device__ __forceinline__ void load_row_to_lds(__amdgpu_buffer_rsrc_t r, void* 
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16, voffset, soffset, 0, 0);
 }
 
-// Clock stamps per wave for profiling builds; nothing otherwise.  A profiling build compiles a
-// kernel source with -DTMX_PROF_STAMPS, points g_stamps (hipMemcpyToSymbol) at a zeroed device
-// array of [workgroups][waves per workgroup][32] 64-bit slots and reads it back after the launch:
-// slot i of a wave holds the 100 MHz wall clock at TMX_STAMP(i).  The kernel needs `lane` and
-// `wave` in scope.  This is how the phase times quoted in the kernels' comments were taken.
-#ifdef TMX_PROF_STAMPS
-__device__ unsigned long long* g_stamps;  // [workgroup][wave][32]
-#define TMX_STAMP(i)                                                                              \
-  if (g_stamps && lane == 0)                                                                      \
-  g_stamps[((size_t)blockIdx.x * (blockDim.x >> 6) + wave) * 32 + (i)] = wall_clock64()
-#else
-#define TMX_STAMP(i)
-#endif
 
 inline int check_launch() {
   hipError_t e = hipGetLastError();

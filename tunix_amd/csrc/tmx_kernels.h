@@ -147,7 +147,7 @@ struct HeadArgs {
   const int32_t* forbidden;
   int n_forbidden;
   float* logits_out;  // [M, V] raw f32 logits, optional
-  uint64_t* sort_keys;  // [M, V] (row << 32) | ~ordered(z): set for the sorting (nucleus / top-k) branch
+  uint16_t* sort_keys;  // [M, V] 16-bit descending key of every bf16 logit: set for the nucleus / top-k branch
   float* part_f;      // [M][nwg][4] = max, sumexp, best key, best z
   int32_t* part_i;    // [M][nwg]
   int nwg;
@@ -166,8 +166,11 @@ struct HeadArgs {
 
 
 struct NucleusArgs {
-  const uint64_t* keys;  // [M, V] sorted ascending
-  const uint32_t* vals;  // [M, V] linear index row * V + v of each sorted key
+  const uint16_t* keys;  // [M, V] 16-bit descending keys of the bf16 logits (written by the head kernel)
+  uint32_t* ent;         // [M][2 halves][3][32768]: key value | count prefix | mass prefix (f32 bits) of the populated values
+  uint32_t* tot;         // [M][2][4]: populated values, candidates, mass (f32 bits), row maximum of z (f32 bits)
+  float* pbest;          // [M][ns][4]: noisy key, z, rank (int bits) of each slice's winner
+  int ns;                // slices of the rank range per row
   int M, V, k;           // k: candidates kept by top-k (V without top-k)
   float top_p;
   float temperature;     // the keys order the bf16 logits; z = logit / temperature
