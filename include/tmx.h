@@ -107,6 +107,19 @@ int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight, co
                             const void* lora_a_t, float* y_part, float* t_part, int M, int K, int N,
                             int G, int r_pad, int nsplit);
 
+/* One projection of the single-sequence regime (1..4 rows) in ONE launch: optional RMSNorm of
+ * x in the prologue (norm_w != NULL; family as tmx_rmsnorm), the int4 product, the LoRA delta
+ * computed inside (t = x . A by every workgroup), then either nothing, the residual add
+ * y = bf16(y + residual), or SwiGLU (swiglu != 0: N = 2 F stacked gate | up columns, y is
+ * [M, F] = bf16(silu(gate) * up), r_pad == 32 with 2 r <= 32).  Same rounding chain as
+ * tmx_rmsnorm + tmx_qlora_linear (+ tmx_swiglu).  M <= 4, M K <= 16384 with the norm (32768
+ * without), r <= 32, r_pad <= 64; the norm and the residual do not combine.
+ * tunix/models/llama3/model.py:290-297, :216-218, :489-496, :546-564. */
+int tmx_small_linear(void* stream, const void* x, const void* norm_w, float eps, int family,
+                     const void* qweight, const void* scales, const void* lora_a_t, const void* lora_b,
+                     const void* residual, void* y, int M, int K, int N, int G, int r, int r_pad,
+                     float lora_scale, int swiglu);
+
 /* ---- row-wise kernels between the matrix products ------------------------- */
 
 /* y[M, D] = RMSNorm(x) * w.  TMX_FAMILY_LLAMA3: bf16(bf16(w * x) / rms)

@@ -671,3 +671,75 @@ def test_moe_experts_match_oracle(B, D, F, E, k, group):
     acc_err = 2.0 ** -23 * (np.abs(got_act[rows]) @ np.abs(ld.weight()))
     G.assert_bf16_close(got_y[rows], want_y, ulps=1.0, extra=acc_err, min_exact=0.995, what=f'down e{e}', stragglers=few)
   assert not np.isin(idx, E - 1).any()
+
+
+# ---- single-sequence regime: norm | projection | LoRA | residual / SwiGLU in one launch -----------
+
+@pytest.mark.parametrize('M,K,N,group,r,mode', [
+    (1, 2048, 3072, 64, 16, 'norm'), (1, 2048, 2048, 64, 16, 'residual'), (1, 2048, 1024, 64, 16, 'swiglu'),
+    (1, 8192, 2048, 64, 16, 'residual'), (4, 256, 96, 64, 8, 'norm'), (3, 512, 256, 128, 0, 'plain'),
+    (2, 1024, 256, 64, 32, 'residual'), (4, 512, 128, 64, 4, 'swiglu'), (1, 320, 64, 64, 0, 'swiglu'),
+    (1, 2048, 3072, 64, 0, 'norm_qwen')])
+def test_small_linear_matches_oracle(M, K, N, group, r, mode):
+  T = G.Keep()
+  rng = np.random.default_rng(M * 13 + K + N)
+  w = bf16_round(rng.standard_normal((K, N)).astype(np.float32) * 0.02)
+  x = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+  res = bf16_round(rng.standard_normal((M, N)).astype(np.float32))
+  nw = bf16_round(1.0 + 0.1 * rng.standard_normal(K).astype(np.float32))
+  swiglu = mode == 'swiglu'
+  a = b = None
+  loras = None
+  if r:
+    a = bf16_round(rng.standard_normal((K, r)).astype(np.float32) * 0.02)
+    b = bf16_round(rng.standard_normal((r, N)).astype(np.float32) * 0.02)
+  if swiglu:
+    F = N // 2
+    ws = [w[:, :F], w[:, F:]]
+    # gate and up carry their own A (the same values here) and their own B columns
+    pl = quant.PackedLinear.from_dense([torch.from_numpy(np.ascontiguousarray(v)) for v in ws], group, G.DEV,
+                                       [(torch.from_numpy(a), torch.from_numpy(np.ascontiguousarray(b[:, :F]))),
+                                        (torch.from_numpy(a), torch.from_numpy(np.ascontiguousarray(b[:, F:])))] if r else None, 2.0)
+  else:
+    pl = _packed(w, group, (a, b) if r else None, 2.0)
+  qo, so = int4.quantize(w, group)
+  lin = L.Linear(q=qo, scale=so, group=group, a=a, b=b, lora_scale=2.0)
+  family = 1 if mode == 'norm_qwen' else 0
+  use_norm = mode in ('norm', 'norm_qwen', 'swiglu')
+  xin = x
+  if use_norm:
+    xin = (L.rmsnorm_qwen3 if family else L.rmsnorm_llama3)(x, nw, 1e-5, BF16)
+  out = lin(xin, BF16)
+  base = bf16_round(xin @ lin.weight())
+  if swiglu:
+    F = N // 2
+    want = bf16_round(L.silu(out[:, :F], BF16) * out[:, F:])
+  elif mode == 'residual':
+    want = bf16_round(out + res)
+  else:
+    want = out
+  y = torch.full(want.shape, float('nan'), dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_small_linear', S(), T.bf(x), T.bf(nw) if use_norm else None, 1e-5, family, G.p(pl.qweight), G.p(pl.scales),
+         G.p(pl.lora_a_t), G.p(pl.lora_b), T.bf(res) if mode == 'residual' else None, G.p(y), M, K, N, group, r,
+         pl.r_pad, 2.0, 1 if swiglu else 0)
+  G.sync()
+  got = G.host(y)
+  if swiglu:
+    # a last-bit flip of gate or up (f32 summation order) moves the product by about an ulp of it
+    G.assert_bf16_close(got, want, ulps=2.0, extra=1e-6 + 2.0 * G.ulp_bf16(want), min_exact=0.97, what=f'small swiglu {K}x{N}')
+  else:
+    extra = (G.ulp_bf16(base) + G.ulp_bf16(out)) if (r or mode == 'residual') else 0.0
+    if r:
+      extra = extra + 2.0 * G.ulp_bf16(out - base)
+    extra = extra + 2.0 ** -23 * (np.abs(xin) @ np.abs(lin.weight()))
+    G.assert_bf16_close(got, want, ulps=1.0, extra=extra, min_exact=0.99, what=f'small {mode} {M}x{K}x{N}')
+
+
+def test_small_linear_rejects_what_it_cannot_take():
+  lib = _lib.lib()
+  one = torch.zeros(64, dtype=torch.uint8, device=G.DEV)
+  p = G.p(one)
+  assert lib.tmx_small_linear(S(), p, None, 1e-5, 0, p, p, None, None, None, p, 5, 256, 64, 64, 0, 0, 0.0, 0) == -2   # 5 rows
+  assert lib.tmx_small_linear(S(), p, p, 1e-5, 0, p, p, None, None, None, p, 4, 8192, 64, 64, 0, 0, 0.0, 0) == -2  # M K too large for the norm
+  assert lib.tmx_small_linear(S(), p, None, 1e-5, 0, p, p, None, None, None, p, 1, 256, 64, 64, 0, 0, 0.0, 1) == -4  # SwiGLU needs the norm prologue
+  assert lib.tmx_small_linear(S(), None, None, 1e-5, 0, p, p, None, None, None, p, 1, 256, 64, 64, 0, 0, 0.0, 0) == -1

@@ -18,6 +18,7 @@ SIGNATURES = {
     'tmx_int4_dequant': [vp, vp, vp, vp, ci, ci, ci],
     'tmx_qlora_linear': [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
     'tmx_qlora_linear_noalloc': [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
+    'tmx_small_linear': [vp, vp, vp, cf, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf, ci],
     'tmx_qlora_linear_num_splits': [ci, ci, ci],
     'tmx_qlora_linear_num_lora_splits': [ci, ci],
     'tmx_qlora_linear_planes': [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci],

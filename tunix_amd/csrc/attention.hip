@@ -18,22 +18,6 @@
 
 namespace tmx {
 
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-  return __builtin_bit_cast(
-      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
-}
-// Sum over aligned groups of LPP (8 or 16) lanes; every lane gets the total.
-template <int LPP>
-__device__ __forceinline__ float group_sum(float v) {
-  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
-  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
-  v += dpp_f<0x141>(v);  // row_half_mirror
-  if (LPP == 16) v += dpp_f<0x140>(v);  // row_mirror
-  return v;
-}
-
-
 // waves per workgroup: fewer for wide groups so the merge buffers stay under 64 KiB
 template <int G>
 struct AttnWaves { static constexpr int value = G > 4 ? 2 : 4; };

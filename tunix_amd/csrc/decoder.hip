@@ -20,6 +20,9 @@ struct Workspace {
   uint16_t *x, *xn, *q, *attn, *act, *y16;
   float *y_part, *t_part, *rope_tab;
   uint16_t* t16;  // bf16 LoRA projection of a many-rows pass
+  void* gu_sync;  // hand-over area of the fused gate | up launch (LoRA projection computed once per launch)
+  float* sb_tparts;        // small-batch step: parts of the down projection's t left by gate | up
+  float* sb_attn_partial;  // small-batch step: split results of the attention kernel
   float* attn_partial;
   void* head_partial;
   // routed experts (MoE models)
@@ -34,6 +37,31 @@ struct Workspace {
 static const int kFusedGateUpMaxRows = 64;
 
 struct Splits { int qkv, o, gate_up, down; };
+
+// One to four sequences, one token each, dense Llama-family layers whose shapes fit the small-batch
+// kernels: five launches per layer (see smallbatch.hip).
+static const int kSmallBatchMaxRows = 4;
+static bool small_batch_ok(const tmx_model_desc* m, int B, int T) {
+  if (B > kSmallBatchMaxRows || T != 1 || m->num_experts > 0 || m->family != TMX_FAMILY_LLAMA3) return false;
+  const int D = m->embed_dim, N = m->num_heads, Kh = m->num_kv_heads, H = m->head_dim, F = m->hidden_dim;
+  const int NH = N * H, QKV = (N + 2 * Kh) * H;
+  if (!sb_attn_ok(N, Kh, H)) return false;
+  for (int i = 0; i < m->num_layers; ++i) {
+    const tmx_layer_desc& l = m->layers[i];
+    if (l.q_norm_w || l.k_norm_w) return false;
+    if (!sb_linear_ok(B, D, QKV, l.qkv.G, l.qkv.lora_a_t ? l.qkv.rank : 0, l.qkv.lora_a_t ? l.qkv.r_pad : 0, true)) return false;
+    if (!sb_linear_ok(B, NH, D, l.o.G, l.o.lora_a_t ? l.o.rank : 0, l.o.lora_a_t ? l.o.r_pad : 0, false)) return false;
+    if (F % 32 || !sb_linear_ok(B, D, 2 * F, l.gate_up.G, l.gate_up.lora_a_t ? l.gate_up.rank : 0,
+                                l.gate_up.lora_a_t ? l.gate_up.r_pad : 0, true))
+      return false;
+    if (!sb_linear_ok(B, F, D, l.down.G, l.down.lora_a_t ? l.down.rank : 0, l.down.lora_a_t ? l.down.r_pad : 0, false))
+      return false;
+    if (l.qkv.lora_a_t && 3 * l.qkv.rank > 64) return false;
+    if (l.gate_up.lora_a_t && (l.gate_up.r_pad != 32 || 2 * l.gate_up.rank > 32)) return false;
+    if (l.down.lora_a_t && l.down.r_pad != 32) return false;
+  }
+  return true;
+}
 
 static Splits plan_splits(const tmx_model_desc* m, int B) {
   const int D = m->embed_dim, NH = m->num_heads * m->head_dim;
@@ -72,6 +100,10 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   w.y_part = (float*)take((size_t)B * ypart * 4);
   w.t_part = (float*)take((size_t)TMX_MAX_LORA_SPLITS * B * TMX_MAX_RPAD * 4);
   w.t16 = (uint16_t*)take(B > 128 ? (size_t)B * TMX_MAX_RPAD * 2 : 0);
+  w.gu_sync = take(B <= kFusedGateUpMaxRows && m->num_experts == 0 && D % 256 == 0 ? qlinear_gate_up_sync_bytes(B, (int)D) : 0);
+  const bool small = B <= kSmallBatchMaxRows && m->num_experts == 0;
+  w.sb_tparts = (float*)take(small ? (F / 32 + 1) * (size_t)B * 32 * 4 : 0);
+  w.sb_attn_partial = (float*)take(small ? sb_attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C) : 0);
   w.rope_tab = (float*)take((size_t)B * m->head_dim * 4);
   w.attn_partial = (float*)take(attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C));
   w.head_partial = take(head_partial_bytes(B, m->vocab_size));
@@ -163,6 +195,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
   }
 
   const Splits sp = plan_splits(m, B);
+  const bool small = small_batch_ok(m, B, T);
   auto lora_of = [&](const tmx_qlinear_desc& l, int) {
     LoraIn li = {};
     if (l.lora_a_t) {
@@ -183,6 +216,11 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     return qlinear_wide_lora(st, x, ldx, l.qweight, l.scales, l.lora_a_t, l.lora_b, l.rank, l.lora_scale, seg_end,
                              w.y16, w.t_part, w.t16, B, l.K, l.N, l.G, l.r_pad);
   };
+  // the hand-over words of the fused gate | up launch start at zero (the kernel leaves them so)
+  if (!moe && B <= kFusedGateUpMaxRows && w.gu_sync && n_steps > 0) {
+    rc = zero_words(st, (uint32_t*)w.gu_sync, 64);
+    if (rc != TMX_OK) return rc;
+  }
   for (int it = 0; it < n_steps; ++it) {
     {  // embedding gather + first input norm + this step's RoPE table
       RowNormArgs a = {};
@@ -202,7 +240,75 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       a.D = D; a.eps = m->norm_eps; a.family = m->family;
       TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
     }
-    for (int i = 0; i < m->num_layers; ++i) {
+    if (small) {
+      // the residual stream lives in w.x (the embedding row kernel wrote it); norms run inside the projections
+      for (int i = 0; i < m->num_layers; ++i) {
+        const tmx_layer_desc& l = m->layers[i];
+        uint16_t* kc = (uint16_t*)s->kv_cache + (size_t)(2 * i) * kv_elems;
+        uint16_t* vc = kc + kv_elems;
+        auto base_args = [&](const tmx_qlinear_desc& d, bool own_t) {
+          SbLinearArgs a = {};
+          a.M = B;
+          a.eps = m->norm_eps; a.family = m->family;
+          a.qw = (const uint4*)d.qweight; a.scales = (const uint16_t*)d.scales;
+          a.K = d.K; a.N = d.N; a.G = d.G;
+          a.seg_end[0] = a.seg_end[1] = a.seg_end[2] = d.N;
+          if (d.lora_a_t) {
+            if (own_t) { a.a_t = (const uint16_t*)d.lora_a_t; a.Rpad = d.r_pad; }
+            a.lora_b = (const uint16_t*)d.lora_b; a.lora_r = d.rank; a.lora_ls = d.lora_scale;
+          }
+          a.ldy = d.N;
+          return a;
+        };
+        {
+          SbLinearArgs a = base_args(l.qkv, true);
+          a.x = w.x; a.ldx = D; a.norm_w = (const uint16_t*)l.norm1_w;
+          a.seg_end[0] = NH; a.seg_end[1] = NH + Kh * H;
+          a.y = w.y16;
+          TMX_TRY(TMX_K_QKV, sb_linear(st, a, 1, 0));
+        }
+        const int ans = sb_attn_splits(B, Kh, C);
+        {
+          SbAttnArgs a = {};
+          a.qkv = w.y16; a.rope_tab = w.rope_tab; a.kcache = kc; a.vcache = vc;
+          a.input_mask = s->input_mask; a.step = s->step; a.buf_len = L;
+          a.partial = w.sb_attn_partial;
+          a.B = B; a.N = N; a.Kh = Kh; a.C = C; a.nsplit = ans;
+          a.scale = 1.0f / sqrtf((float)H);
+          TMX_TRY(TMX_K_ATTN, sb_attn(st, a, H));
+        }
+        {
+          SbLinearArgs a = base_args(l.o, true);
+          a.attn_part = w.sb_attn_partial; a.attn_kh = Kh; a.attn_g = N / Kh; a.attn_h = H; a.attn_ns = ans;
+          a.residual = w.x; a.y = w.x;
+          TMX_TRY(TMX_K_O, sb_linear(st, a, 2, 1));
+        }
+        {
+          SbLinearArgs a = base_args(l.gate_up, true);
+          a.x = w.x; a.ldx = D; a.norm_w = (const uint16_t*)l.norm2_w;
+          a.seg_end[0] = F;
+          a.y = w.act; a.ldy = F; a.pair_off = F / 32;
+          if (l.down.lora_a_t) { a.a_next = (const uint16_t*)l.down.lora_a_t; a.t_parts_out = w.sb_tparts; }
+          TMX_TRY(TMX_K_GATE_UP, sb_linear(st, a, 1, 2));
+        }
+        {
+          SbLinearArgs a = base_args(l.down, false);
+          a.x = w.act; a.ldx = F;
+          if (l.down.lora_a_t) { a.t_parts = w.sb_tparts; a.t_nparts = F / 32; }
+          a.residual = w.x; a.y = w.x;
+          TMX_TRY(TMX_K_DOWN, sb_linear(st, a, 0, 1));
+        }
+        if (prof) TMX_TRY(TMX_K_EMPTY, empty_launch(st));
+      }
+      {  // final norm in front of the head
+        RowNormArgs a = {};
+        a.y_bf16 = w.x;
+        a.norm_w = (const uint16_t*)m->final_norm_w; a.xn_out = w.xn;
+        a.D = D; a.eps = m->norm_eps; a.family = m->family;
+        if (sample) TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
+      }
+    }
+    for (int i = 0; !small && i < m->num_layers; ++i) {
       const tmx_layer_desc& l = m->layers[i];
       // gate | up with LoRA + SwiGLU in its epilogue: K % 256 == 0 below 8192, unsplit, 2 r <= 32
       const bool fused_gu = !moe && B <= kFusedGateUpMaxRows && sp.gate_up == 1 && D % 256 == 0 && D < 8192 && F % 64 == 0 &&
@@ -306,7 +412,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         if (fused_gu) {
           TMX_TRY(TMX_K_GATE_UP, qlinear_gate_up_swiglu(
               st, w.xn, D, l.gate_up.qweight, l.gate_up.scales, l.gate_up.lora_a_t, l.gate_up.lora_b,
-              l.gate_up.rank, l.gate_up.lora_scale, w.act, B, D, F, l.gate_up.G));
+              l.gate_up.rank, l.gate_up.lora_scale, w.act, B, D, F, l.gate_up.G, w.gu_sync));
         } else {
         const bool gu16 = sp.gate_up == 1;
         {

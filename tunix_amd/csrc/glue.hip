@@ -557,6 +557,16 @@ int advance_step(hipStream_t st, int32_t* step, int by) {
   return check_launch();
 }
 
+__global__ void zero_words_kernel(uint32_t* p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+int zero_words(hipStream_t st, uint32_t* p, int n) {
+  hipLaunchKernelGGL(zero_words_kernel, dim3((n + 255) / 256), dim3(256), 0, st, p, n);
+  return check_launch();
+}
+
 __global__ void empty_kernel() {}
 
 int empty_launch(hipStream_t st) {

@@ -798,17 +798,111 @@ struct GU8 {
 
 
 
-template <int MT, bool FUSE>
+// LoRA inside the gate | up launch, two ways.  LORA == 1: every workgroup multiplies x by [A_gate | A_up]
+// itself (one extra MFMA group and one extra 4 KiB tile per wave and step).  LORA == 2: the first
+// a.sync_blocks workgroups of the launch compute t = x . A once (a K-slice of 4 k-tiles each, partial
+// tiles added by the last one to arrive) and hand it to the others through memory: every store of the
+// hand-over is a write-through store (sc1) followed by a wait for its completion, the arrival counter
+// and the ready flag are device-scope atomics, and the readers load with sc1, so nothing depends on
+// the per-XCD L2 caches being written back or invalidated inside the kernel.  The main workgroups need
+// t only in their epilogue, long after the producers are done; their wait is bounded (a.sync[3] is set
+// and t taken as zero if the flag never comes).  The last reader puts the three counters back to zero,
+// so the state is all-zero between launches (also under graph replay).
+__device__ __forceinline__ void sc1_store_b128(__amdgpu_buffer_rsrc_t r, u32x4_t v, int off) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, 0x10);
+}
+__device__ __forceinline__ u32x4_t sc1_load_b128(__amdgpu_buffer_rsrc_t r, int off) {
+  return __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0x10));
+}
+
+template <int MT>
+__device__ __forceinline__ void lora_producer_block(const QLinearArgs& a, float* red /* [8][16][64] */) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, nl = lane & 31;
+  const int slice = blockIdx.x, P = a.sync_blocks;
+  constexpr int WM = 8 / MT;            // waves per row tile: each takes one k-tile of the slice
+  const int m = wave / WM, kt = slice * WM + wave % WM;  // host: K / 64 == P * WM
+  const int row = min(m * 32 + nl, a.M - 1);
+  f32x16_t acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  u32x4_t xa[4], at[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    xa[t] = *reinterpret_cast<const u32x4_t*>(a.x + (size_t)row * a.ldx + kt * 64 + t * 16 + h * 8);
+    at[t] = reinterpret_cast<const u32x4_t*>(a.a_t)[(size_t)(kt * 4 + t) * 64 + lane];
+  }
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, xa[t]), __builtin_bit_cast(bf16x8_t, at[t]),
+                                                  acc, 0, 0, 0);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) red[((wave * 16 + r) << 6) + lane] = acc[r];
+  __syncthreads();
+  // partial tile of the slice: the WM k-tile waves of each row tile added in wave order, kept in
+  // accumulator layout [m][r][lane]
+  const __amdgpu_buffer_rsrc_t rp = make_rsrc(a.sync_part, (uint32_t)P * MT * 4096u);
+  const __amdgpu_buffer_rsrc_t rt = make_rsrc(a.sync_t16, (uint32_t)MT * 32 * 64u);
+  constexpr int VPT = MT * 1024 / 512 / 4;  // 16-byte groups per thread (MT == 2: one, MT == 1: every other thread)
+  const int e0 = tid * 4;                    // element index in [m][r][lane], 4 adjacent lanes
+  const bool mine = e0 < MT * 1024;
+  (void)VPT;
+  if (mine) {
+    const int mm = e0 >> 10, rest = e0 & 1023;
+    f32x4_t v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < WM; ++w) {
+      const f32x4_t p = *reinterpret_cast<const f32x4_t*>(red + (((mm * WM + w) * 16) << 6) + rest);
+      v += p;
+    }
+    sc1_store_b128(rp, __builtin_bit_cast(u32x4_t, v), (slice * MT * 1024 + e0) * 4);
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // the write-through stores are complete
+  __syncthreads();
+  __shared__ uint32_t s_old;
+  if (tid == 0) s_old = __hip_atomic_fetch_add(a.sync + 0, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (s_old != (uint32_t)(P - 1)) return;
+  // the last slice to arrive: t = bf16(sum of the partial tiles in slice order), row-major [rows][32]
+  if (mine) {
+    const int mm = e0 >> 10, r = (e0 & 1023) >> 6, l0 = e0 & 63;
+    f32x4_t v = {0.f, 0.f, 0.f, 0.f};
+    for (int sl = 0; sl < P; ++sl)
+      v += __builtin_bit_cast(f32x4_t, sc1_load_b128(rp, (sl * MT * 1024 + e0) * 4));
+    // lanes l0 .. l0 + 3 share h and hold 4 adjacent columns of one row
+    const int trow = mm * 32 + acc_row(r, l0), col = l0 & 31;
+    const uint32_t lo = pack_bf2(v[0], v[1]), hi = pack_bf2(v[2], v[3]);
+    __builtin_amdgcn_raw_buffer_store_b32(lo, rt, (trow * 32 + col) * 2, 0, 0x10);
+    __builtin_amdgcn_raw_buffer_store_b32(hi, rt, (trow * 32 + col + 2) * 2, 0, 0x10);
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (tid == 0) {
+    __hip_atomic_store(a.sync + 0, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(a.sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <int MT, int LORA>
 __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a) {
   using S = GU8<MT>;
+  constexpr bool FUSE = LORA == 1, SYNC = LORA == 2;
   constexpr int TS = S::TS, TPW = S::TPW, XS = S::XS, ROWS = S::ROWS;
   extern __shared__ __align__(16) uint16_t smem[];
+  if constexpr (SYNC) {
+    if ((int)blockIdx.x < a.sync_blocks) {
+      lora_producer_block<MT>(a, reinterpret_cast<float*>(smem));
+      return;
+    }
+  }
+  const int bx = SYNC ? (int)blockIdx.x - a.sync_blocks : (int)blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), cw = wave & 3, kh = wave >> 2;
   const int h = lane >> 5, nl = lane & 31;
   const int KT = a.K >> 6, nsteps = KT / TS, last_step = nsteps - 1;  // host: K % (64 TS) == 0
   const int gs = __builtin_ctz(a.G >> 6), KG = a.K / a.G;
-  const int nb = (int)blockIdx.x * 2 + (cw & 1) + (cw >> 1) * a.pair_off;  // host: F % 64 == 0
+  const int nb = bx * 2 + (cw & 1) + (cw >> 1) * a.pair_off;  // host: F % 64 == 0
 
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qw, (uint32_t)(a.N >> 5) * KT * 1024u);
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scales, (uint32_t)(a.N >> 5) * KG * 64u);
@@ -820,7 +914,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   // LoRA B values of this tile's columns for the epilogue (rows h * 8 .. + 7 of B): read now, so
   // that the cold reads complete under the main loop
   uint16_t tbv[8];
-  if constexpr (FUSE) {
+  if constexpr (FUSE || SYNC) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int k = h * 8 + j;
@@ -950,17 +1044,43 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   float* hb = fl + 8 * MT * 1024;
   uint16_t* ts = reinterpret_cast<uint16_t*>(fl + 12 * MT * 1024);
   bf16x8_t tb;
-  if constexpr (FUSE) {
+  if constexpr (FUSE || SYNC) {
     // B fragment of this tile's columns: rows beyond the rank are zero, which also masks the t
     // columns of the other projection inside the 16-wide k window
     uint16_t bz[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) bz[j] = (h * 8 + j) < a.lora_r ? tbv[j] : (uint16_t)0;
     __builtin_memcpy(&tb, bz, 16);
+  }
+  if constexpr (FUSE) {
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int r = 0; r < 16; ++r) fl[(((wave * MT + m) * 16 + r) << 6) + lane] = tacc[m][r];
+  }
+  bf16x8_t tsync[MT];
+  if constexpr (SYNC) {
+    // t from the producer workgroups: wait (bounded) for the ready flag, then read the rows this
+    // lane needs as MFMA A fragments with loads that bypass this XCD's L2
+    __shared__ uint32_t s_ready;
+    if (tid == 0) {
+      uint32_t ok = 0;
+      for (int spin = 0; spin < (1 << 20); ++spin) {
+        if (__hip_atomic_load(a.sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) { ok = 1; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      if (!ok) __hip_atomic_store(a.sync + 3, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_ready = ok;
+    }
+    __syncthreads();
+    const __amdgpu_buffer_rsrc_t rt = make_rsrc(a.sync_t16, (uint32_t)MT * 32 * 64u);
+    const int toff = (cw >= 2) ? a.lora_r : 0;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (s_ready) v = sc1_load_b128(rt, ((m * 32 + nl) * 32 + toff + h * 8) * 2);
+      tsync[m] = __builtin_bit_cast(bf16x8_t, v);
+    }
   }
   // the two k-halves of a tile swap halves of their accumulators: the first half finishes
   // registers 0..7, the second 8..15 (a + b == b + a: the sum does not depend on who adds)
@@ -1003,11 +1123,12 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
         __builtin_memcpy(&ta, tv, 16);
         dl = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta, tb, dl, 0, 0, 0);
       }
+      if constexpr (SYNC) dl = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tsync[m], tb, dl, 0, 0, 0);
 #pragma unroll
       for (int r8 = 0; r8 < 8; ++r8) {
         const int r = kh ? r8 + 8 : r8;
         float y = rbf((kh ? acc[m][r8 + 8] : acc[m][r8]) + hb[(((cw * MT + m) * 16 + r) << 6) + lane]);
-        if (FUSE) y = rbf(y + rbf(rbf(kh ? dl[r8 + 8] : dl[r8]) * a.lora_ls));
+        if (FUSE || SYNC) y = rbf(y + rbf(rbf(kh ? dl[r8 + 8] : dl[r8]) * a.lora_ls));
         fl[(((cw * MT + m) * 16 + r) << 6) + lane] = y;  // partial tiles were consumed before the last barrier
       }
     }
@@ -1016,7 +1137,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
   // act = bf16(bf16(g * bf16(sigmoid(g))) * u): every wave finishes a quarter of one gate tile
   {
     const int gt = wave & 1, q = wave >> 1;
-    const int col = ((int)blockIdx.x * 2 + gt) * 32 + nl;
+    const int col = (bx * 2 + gt) * 32 + nl;
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -1030,16 +1151,28 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
         a.y_bf16[(size_t)row * a.ldy + col] = f2bf(rbf(g * sg) * u);
       }
   }
+  if constexpr (SYNC) {
+    // every lane's t fragments were consumed before the barrier above; the last reader of the launch
+    // puts the hand-over state back to zero
+    if (tid == 0) {
+      const uint32_t old = __hip_atomic_fetch_add(a.sync + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (old == (uint32_t)(a.n_main_blocks - 1)) {
+        __hip_atomic_store(a.sync + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(a.sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
 }
 
-template <int MT, bool FUSE>
+template <int MT, int LORA>
 static int launch_gate_up8(hipStream_t st, const QLinearArgs& a) {
   using S = GU8<MT>;
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&qlinear_gate_up8_kernel<MT, FUSE>),
+      reinterpret_cast<const void*>(&qlinear_gate_up8_kernel<MT, LORA>),
       hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS);
   if (attr != hipSuccess) return TMX_ERR_LAUNCH;
-  hipLaunchKernelGGL((qlinear_gate_up8_kernel<MT, FUSE>), dim3(a.n_main_blocks, 1), dim3(512), S::LDS, st, a);
+  const int blocks = a.n_main_blocks + (LORA == 2 ? a.sync_blocks : 0);
+  hipLaunchKernelGGL((qlinear_gate_up8_kernel<MT, LORA>), dim3(blocks, 1), dim3(512), S::LDS, st, a);
   return check_launch();
 }
 
@@ -1566,9 +1699,15 @@ static int lora_slice_len(int K, int N) {
 // gate | up projection with the LoRA deltas and SwiGLU in the epilogue: act[M, F] =
 // bf16(silu(gate) * up).  Needs the 4-wave kernel (K % 256 == 0, K < 8192) and F % 64 == 0;
 // with LoRA: a_t = [A_gate | A_up] in fragment order with r_pad == 32 (2 r <= 32), lora_b [r][2 F].
+size_t qlinear_gate_up_sync_bytes(int M, int K) {
+  // hand-over state (4 words, 256 bytes reserved) | partial tiles [K / 256][rows / 32][16][64] f32 | t bf16 [rows][32]
+  const size_t mt = M <= 32 ? 1 : 2;
+  return 256 + (size_t)(K / 256) * mt * 4096 + mt * 32 * 64;
+}
+
 int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
-                           int F, int G) {
+                           int F, int G, void* sync_ws) {
   if (!x || !qw || !scales || !act) return TMX_ERR_ARG;
   if (M <= 0 || M > 128 || !four_wave_shape(K) || F % 64 || G % 64 || (G & (G - 1)) || K % G || ldx % 8)
     return TMX_ERR_SHAPE;
@@ -1598,8 +1737,19 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
   // up to 64 rows: 8 waves per workgroup, when steps of 8 k-tiles divide K and 32-bit byte
   // offsets reach every operand (128 rows would not fit the register file at 2 waves per SIMD)
   if (M <= 64 && K % 512 == 0 && (size_t)M * ldx * 2 < (1u << 31) && (size_t)K * F < (1u << 31)) {
-    if (a_t) return M <= 32 ? launch_gate_up8<1, true>(st, a) : launch_gate_up8<2, true>(st, a);
-    return M <= 32 ? launch_gate_up8<1, false>(st, a) : launch_gate_up8<2, false>(st, a);
+    if (a_t && sync_ws && K / 256 <= 32 && a.n_main_blocks + K / 256 <= 256) {
+      // t = x . A by K / 256 extra workgroups of the launch, handed to the others through memory; every
+      // workgroup must be resident at once (one per CU), or a main workgroup could wait for a producer
+      // that has no CU to run on
+      const int mt = M <= 32 ? 1 : 2;
+      a.sync = (uint32_t*)sync_ws;
+      a.sync_part = (float*)((char*)sync_ws + 256);
+      a.sync_t16 = (uint16_t*)((char*)sync_ws + 256 + (size_t)(K / 256) * mt * 4096);
+      a.sync_blocks = mt == 1 ? K / 512 : K / 256;  // 8 / MT k-tiles per producer
+      return M <= 32 ? launch_gate_up8<1, 2>(st, a) : launch_gate_up8<2, 2>(st, a);
+    }
+    if (a_t) return M <= 32 ? launch_gate_up8<1, 1>(st, a) : launch_gate_up8<2, 1>(st, a);
+    return M <= 32 ? launch_gate_up8<1, 0>(st, a) : launch_gate_up8<2, 0>(st, a);
   }
   if (a_t) {
     if (M <= 32) return launch(qlinear_gate_up_kernel<1>);
@@ -1870,5 +2020,5 @@ extern "C" int tmx_qlora_gate_up_swiglu(void* stream, const void* x, const void*
                                         const void* lora_a_t, const void* lora_b, void* act, int M, int K,
                                         int F, int G, int r, float lora_scale) {
   return qlinear_gate_up_swiglu((hipStream_t)stream, x, K, qweight, scales, lora_a_t, lora_b, r, lora_scale, act,
-                                M, K, F, G);
+                                M, K, F, G, nullptr);
 }

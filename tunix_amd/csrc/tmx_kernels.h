@@ -32,6 +32,12 @@ struct QLinearArgs {
   const uint16_t* t16;
   int ldt16;
   int seg_end[3];
+  // LoRA projection computed once per launch by extra workgroups and handed over through memory
+  // (fused gate | up kernel): hand-over state {arrivals, ready, readers, timeout}, partial tiles, t
+  uint32_t* sync;
+  float* sync_part;
+  uint16_t* sync_t16;
+  int sync_blocks;
 };
 
 // Routed experts (Qwen3 MoE): one launch multiplies, for every expert, the rows routed to it.
@@ -186,6 +192,55 @@ struct NucleusArgs {
   int buf_len;
 };
 
+// One projection of the small-batch step (1..4 rows): prologue | int4 product + LoRA | epilogue in one launch.
+struct SbLinearArgs {
+  int M;
+  const uint16_t* x;        // plain: activations [M, K]; norm: residual stream [M, K], normalised in the prologue
+  int ldx;
+  const uint16_t* norm_w;   // [K] (norm prologue)
+  float eps;
+  int family;
+  const float* attn_part;   // attention prologue: [M][kh][ns][g][h + 2] split results (output | max | sum)
+  int attn_kh, attn_g, attn_h, attn_ns;
+  const uint4* qw;
+  const uint16_t* scales;
+  int K, N, G;
+  const uint16_t* a_t;      // LoRA A, fragment order (null: t comes from t_parts, or no LoRA)
+  int Rpad;
+  const uint16_t* lora_b;   // [lora_r][N] (null: no LoRA)
+  int lora_r;
+  float lora_ls;
+  int seg_end[3];           // column ends of the fused matrices; segment s uses t columns s lora_r ..
+  const float* t_parts;     // [t_nparts][M][32] parts of t left by the previous launch (down projection)
+  int t_nparts;
+  const uint16_t* residual; // [M, N] (residual epilogue)
+  uint16_t* y;              // [M, N]; SwiGLU epilogue: act [M, N / 2]
+  int ldy;
+  int pair_off;             // SwiGLU epilogue: tile distance between a gate tile and its up tile (N / 64)
+  const uint16_t* a_next;   // SwiGLU epilogue: A of the next projection (r_pad 32), or null
+  float* t_parts_out;       // [N / 64][M][32]
+};
+
+struct SbAttnArgs {
+  const uint16_t* qkv;      // [B, (N + 2 Kh) H] with the LoRA deltas applied
+  const float* rope_tab;    // [B][H / 2][2] sin, cos of this step
+  uint16_t* kcache;         // [B, C, Kh, H]
+  uint16_t* vcache;
+  const uint8_t* input_mask;
+  const int32_t* step;
+  int buf_len;
+  float* partial;           // [B][Kh][nsplit][G][H + 2]
+  int B, N, Kh, C, nsplit;
+  float scale;
+};
+
+int sb_linear(hipStream_t st, const SbLinearArgs& a, int pro, int epi);  // pro: 0 plain, 1 norm, 2 attention merge; epi: 0 plain, 1 residual, 2 SwiGLU
+bool sb_linear_ok(int M, int K, int N, int G, int rank, int rpad, bool norm);
+int sb_attn(hipStream_t st, SbAttnArgs a, int H);
+bool sb_attn_ok(int N, int Kh, int H);
+int sb_attn_splits(int B, int Kh, int C);
+size_t sb_attn_partial_bytes(int B, int N, int Kh, int H, int C);
+
 int row_norm(hipStream_t st, const RowNormArgs& a, int M);
 int rope_kvwrite(hipStream_t st, const RopeArgs& a, int B);
 int swiglu(hipStream_t st, const SwigluArgs& a, int M);
@@ -205,9 +260,13 @@ size_t nucleus_bytes(int M, int V);
 size_t head_partial_bytes(int M, int V);
 int qlinear_num_splits(int K, int N, int M);
 int qlinear_num_lora_splits(int K, int N);
+// sync_ws: qlinear_gate_up_sync_bytes(M, K) bytes whose first 16 are zero between launches (the kernel
+// leaves them so), or null: then every workgroup multiplies x by A itself
 int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
-                           int F, int G);
+                           int F, int G, void* sync_ws);
+size_t qlinear_gate_up_sync_bytes(int M, int K);
+int zero_words(hipStream_t st, uint32_t* p, int n);  // p[0 .. n) = 0 by a small kernel
 // Many rows (M > 128), unsplit: y_bf16 = bf16(bf16(x . W) + bf16(bf16(t . B) ls)) in one pass, t = bf16(x . A)
 // computed by a LoRA-only launch of the same kernel and a small reduction (t_part: f32 planes, t16: bf16
 // [M][TMX_MAX_RPAD] scratch).  seg_end: column ends of the fused matrices (q | k | v, gate | up), unused
