@@ -252,3 +252,16 @@ def test_token_ids_outside_the_vocabulary_are_rejected_before_the_gpu():
     s.per_token_logps(np.array([[3, 4]]), np.array([[5, v + 7]]))
   with pytest.raises(NotImplementedError, match='echo'):
     s(prompt_token_ids=[[3, 4]], max_generation_steps=2, echo=True, return_logits=True)
+
+
+def test_model_from_state_tree_flattens_before_it_builds(monkeypatch):
+  """QLoRAModel.from_state_tree hands from_state the dotted paths of a nested state (no GPU: from_state is stubbed)."""
+  from tunix_amd.model import QLoRAModel
+  seen = {}
+  monkeypatch.setattr(QLoRAModel, 'from_state', classmethod(lambda cls, cfg, state, **kw: seen.update(state=state, kw=kw) or 'built'))
+  w = np.zeros((4, 2, 3), np.float32)
+  tree = {'layers': {0: {'attn': {'q_proj': {'w': _Var(w), 'w_lora_a': _Var(np.zeros((4, 2), np.float32))}}}},
+          'embedder': {'input_embedding': _Var(np.zeros((8, 4), np.float32))}}
+  assert QLoRAModel.from_state_tree(ModelConfig.toy(), tree, group=64, lora_alpha=8.0, device='cpu') == 'built'
+  assert set(seen['state']) == {'layers.0.attn.q_proj.w', 'layers.0.attn.q_proj.w_lora_a', 'embedder.input_embedding'}
+  assert tuple(seen['state']['layers.0.attn.q_proj.w'].shape) == (4, 2, 3) and seen['kw']['lora_alpha'] == 8.0

@@ -198,6 +198,17 @@ class QLoRAModel:
     return m
 
   @classmethod
+  def from_state_tree(cls, config, tree, group=64, lora_alpha=0.0, device='cuda', bound=7.5):
+    """The same from what a tunix caller holds: nnx.state(model) of a (LoRA-wrapped, not yet
+    quantised) Llama3 / Qwen3 module, its pure-dict dump, or any nested mapping with the
+    reference's path parts ('layers', 0, 'attn', 'q_proj', 'w', ...).  Leaves may be arrays or
+    variable objects with the array in `.value`; the tree is flattened to dotted paths
+    (tunix/rl/utils.py:72-78 to_flat_dict) and quantised like from_state."""
+    from tunix_amd import utils
+    return cls.from_state(config, utils.flatten_state(tree), group=group, lora_alpha=lora_alpha, device=device,
+                          bound=bound)
+
+  @classmethod
   def random_init(cls, config, seed=0, group=64, lora_rank=0, lora_alpha=0.0,
                   lora_targets=_ATTN + _MLP, std=0.02, device='cuda'):
     """Synthetic weights generated layer by layer on the device: every matrix

@@ -252,6 +252,7 @@ class Sampler:
   MAX_FILL_ROWS = 4096  # rows of one cache-fill or scoring pass of a dense model (256-row projection blocks)
 
   MAX_MOE_PAIRS = 8192  # routed (token, expert) pairs of one pass of a MoE model
+  MAX_PASSES_IN_FLIGHT = 64  # passes a walk enqueues before it waits for the stream
 
   def _max_rows(self):
     """Rows one pass can take: more than 128 need the 256-row projection blocks (every attention /
@@ -279,10 +280,16 @@ class Sampler:
     # the head chooses tokens for up to MAX_ROWS rows; scoring takes as many rows as a cache fill
     choose = sample and st['sampling_mode'] != 'score'
     per = min(128, max(1, (self.MAX_ROWS if choose else self._fill_rows()) // b))
+    passes = 0
     while n_tokens > 0:
       t = min(per, n_tokens)
       self.run_steps(st, 1, sample=sample, tokens_per_pass=t)
       n_tokens -= t
+      passes += 1
+      if passes % self.MAX_PASSES_IN_FLIGHT == 0:
+        # bound the queue of pending launches (a pass is a few hundred of them): a walk of
+        # thousands of short passes otherwise leaves tens of thousands of dispatches pending at once
+        torch.cuda.current_stream().synchronize()
 
   def run_steps(self, st, n_steps, sample=True, graph=False, tokens_per_pass=1):
     """Runs n decode-loop iterations on the current stream.  graph=False only enqueues (no host
