@@ -353,7 +353,10 @@ def main():
       if fused:
         lora = gu.lora_a_t is not None
         if batch <= 64 and gu.k % 512 == 0:   # 8 waves per workgroup, activation slab by direct-to-LDS loads
-          sym = f"tmx::qlinear_gate_up8_kernel<{mt}, {'true' if lora else 'false'}>"
+          # LoRA mode: 0 none, 1 every workgroup multiplies x by A itself, 2 a few workgroups do it once and
+          # hand t over (K / 256 <= 32 producers that fit beside the F / 64 main workgroups within 256)
+          mode = 0 if not lora else (2 if gu.k // 256 <= 32 and cfg.hidden_dim // 64 + gu.k // 256 <= 256 else 1)
+          sym = f'tmx::qlinear_gate_up8_kernel<{mt}, {mode}>'
         else:
           sym = f'tmx::qlinear_gate_up_kernel<{mt}>' if lora else f'tmx::qlinear_mfma4_kernel<{mt}>'
         symbols.setdefault(sym, []).append('gate_up_linear')
@@ -372,8 +375,16 @@ def main():
     for cls_name, key in dense:
       sym = f'tmx::qlinear_mfma4_kernel<{mt}>' if four(layer0[key]) else kway_symbol(layer0[key])
       symbols.setdefault(sym, []).append(cls_name)
+    small = batch <= 4 and not cfg.num_experts and cfg.family == 'llama3' and tot_cnt[CLASS_NAMES.index('rope_kvwrite')] == 0
+    if small:
+      # 1..4 rows: five launches per layer, norm / LoRA / residual / SwiGLU inside the projections
+      # (template arguments: prologue 0 plain, 1 norm, 2 attention merge; epilogue 0 plain, 1 residual, 2 SwiGLU)
+      symbols = {'tmx::sb_linear_kernel<1, 0>': ['qkv_linear'], 'tmx::sb_linear_kernel<2, 1>': ['o_linear'],
+                 'tmx::sb_linear_kernel<1, 2>': ['gate_up_linear'], 'tmx::sb_linear_kernel<0, 1>': ['down_linear'],
+                 f'tmx::sb_attn_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention']}
+    symbols.update({} if small else {
+        f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention']})
     symbols.update({
-        f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention'],
         ('tmx::head_wide_kernel' if batch > 128 and top_p >= 1.0 else f'tmx::head_kernel<{min(mt, 2)}>'): ['head_sample'],
         # (65..128 rows: two launches of the 64-row kernel)
     })

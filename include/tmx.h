@@ -39,6 +39,7 @@ extern "C" {
 #define TMX_ERR_LAUNCH (-3)      /* the HIP runtime refused the launch */
 #define TMX_ERR_UNSUPPORTED (-4) /* valid request outside what is implemented */
 #define TMX_ERR_SCRATCH (-5)     /* the request needs more scratch memory than the library's static buffer holds */
+#define TMX_ERR_DEVICE_WAIT (-6) /* a bounded wait inside a kernel ran out (reported by tmx_decode_status) */
 
 #define TMX_FAMILY_LLAMA3 0
 #define TMX_FAMILY_QWEN3 1
@@ -328,6 +329,17 @@ size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int ca
  * `model`, `state` and model->layers are HOST structures read during the call only. */
 int tmx_decode_steps(const tmx_model_desc* model, const tmx_decode_state* state, void* stream,
                      int n_steps, int sample);
+
+/* Some decode kernels hand data from one group of workgroups to another inside a launch (the
+ * fused gate | up projection computes its LoRA projection once and passes it on).  The
+ * receiving side waits a bounded number of polls; if a wait ever runs out the kernel carries
+ * on with zeros and sets a sticky word in the workspace.  This call WAITS for `stream`, reads
+ * that word, clears it, and returns TMX_ERR_DEVICE_WAIT if it was set (the tokens produced
+ * since the previous check are then not to be trusted), else TMX_OK.  The word lives in the
+ * first 256 bytes of state->workspace, which the decode calls never clear: zero-fill them
+ * once before the workspace's first use.  No counterpart in the reference (XLA has no such
+ * failure mode). */
+int tmx_decode_status(const tmx_model_desc* model, const tmx_decode_state* state, void* stream);
 
 /* The same steps with one of them recorded into a HIP graph and replayed n_steps - 1 times
  * (fewer host launches; what the reference gets from jit-compiling the while_loop).  Unlike

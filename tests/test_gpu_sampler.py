@@ -326,6 +326,23 @@ def test_unsupported_sampling_modes_fail_loudly():
     s(input_strings=['5 6'], max_generation_steps=2, beam_size=2)
 
 
+def test_device_status_reports_a_wait_that_ran_out():
+  """tmx_decode_status: clean after a rollout; a set status word (written here from the host, no
+  kernel is made to wait) is reported once as TMX_ERR_DEVICE_WAIT and cleared."""
+  from tunix_amd import _lib
+  cfg = C.TOY
+  _, model = _pair(cfg, seed=16)
+  s = _sampler(model, cfg, 32)
+  s(input_strings=['5 6 7'], max_generation_steps=4)  # checks the status itself before returning
+  st = s.init_sample_state(np.array([[5, 6, 7]], np.int32), 8, False, None, 1.0, 1.0, None, 0, include_logprobs=False)
+  s.run_steps(st, 2, sample=False)
+  s.check_device_status(st)
+  s._workspace[:4] = torch.tensor([1, 0, 0, 0], dtype=torch.uint8, device=s._workspace.device)
+  with pytest.raises(_lib.TmxError, match='bounded wait'):
+    s.check_device_status(st)
+  s.check_device_status(st)  # cleared by the failing check
+
+
 def test_moe_decoder_matches_oracle():
   """Qwen3-MoE-shaped toy (8 experts, top-2, QK-norm): greedy tokens and step logits against
   the oracle's routed-pair restatement of MoELayer (tunix/models/qwen3/model.py:894-939)."""

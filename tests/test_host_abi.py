@@ -36,7 +36,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_status_strings_and_version():
   lib = _lib.lib()
-  assert lib.tmx_abi_version() == 3
+  assert lib.tmx_abi_version() == 4
   assert lib.tmx_status_string(0) == b'ok'
   for code in (-1, -2, -3, -4):
     assert len(lib.tmx_status_string(code)) > 5

@@ -39,6 +39,7 @@ SIGNATURES = {
     'tmx_decode_steps': [vp, vp, vp, ci, ci],
     'tmx_decode_steps_graph': [vp, vp, vp, ci, ci],
     'tmx_decode_steps_profiled': [vp, vp, vp, ci, ci, vp, vp],
+    'tmx_decode_status': [vp, vp, vp],
 }
 # entry points that return size_t
 SIZE_FUNCS = {

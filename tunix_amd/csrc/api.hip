@@ -9,8 +9,9 @@ extern "C" const char* tmx_status_string(int status) {
     case TMX_ERR_LAUNCH: return "HIP launch failed";
     case TMX_ERR_UNSUPPORTED: return "unsupported configuration";
     case TMX_ERR_SCRATCH: return "the request needs more scratch memory than the library's static buffer holds";
+    case TMX_ERR_DEVICE_WAIT: return "a bounded wait inside a kernel ran out: results since the last status check are invalid";
     default: return "unknown status";
   }
 }
 
-extern "C" int tmx_abi_version(void) { return 3; }
+extern "C" int tmx_abi_version(void) { return 4; }

@@ -17,6 +17,7 @@ namespace tmx {
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Workspace {
+  uint32_t* status;  // first 256 bytes, the same place for every batch size: word 0 is set when a bounded wait inside a kernel runs out
   uint16_t *x, *xn, *q, *attn, *act, *y16;
   float *y_part, *t_part, *rope_tab;
   uint16_t* t16;  // bf16 LoRA projection of a many-rows pass
@@ -91,6 +92,7 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   if (sp.o * D > ypart) ypart = sp.o * D;
   if (sp.down * D > ypart) ypart = sp.down * D;
   if (sp.gate_up > 1 && sp.gate_up * 2 * F > ypart) ypart = sp.gate_up * 2 * F;
+  w.status = (uint32_t*)take(256);
   w.x = (uint16_t*)take(B * D * 2);
   w.xn = (uint16_t*)take(B * D * 2);
   w.q = (uint16_t*)take(B * NH * 2);
@@ -412,7 +414,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         if (fused_gu) {
           TMX_TRY(TMX_K_GATE_UP, qlinear_gate_up_swiglu(
               st, w.xn, D, l.gate_up.qweight, l.gate_up.scales, l.gate_up.lora_a_t, l.gate_up.lora_b,
-              l.gate_up.rank, l.gate_up.lora_scale, w.act, B, D, F, l.gate_up.G, w.gu_sync));
+              l.gate_up.rank, l.gate_up.lora_scale, w.act, B, D, F, l.gate_up.G, w.gu_sync, w.status));
         } else {
         const bool gu16 = sp.gate_up == 1;
         {
@@ -519,6 +521,20 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
 extern "C" int tmx_decode_steps(const tmx_model_desc* m, const tmx_decode_state* s, void* stream,
                                 int n_steps, int sample) {
   return decode_steps_impl(m, s, stream, n_steps, sample, nullptr);
+}
+
+extern "C" int tmx_decode_status(const tmx_model_desc* m, const tmx_decode_state* s, void* stream) {
+  if (!m || !s || !s->workspace || !m->layers) return TMX_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  if (s->workspace_bytes < 256) return TMX_ERR_ARG;
+  uint32_t flag = 0;
+  uint32_t* word = (uint32_t*)s->workspace;  // Workspace::status
+  if (hipMemcpyAsync(&flag, word, 4, hipMemcpyDeviceToHost, st) != hipSuccess) return TMX_ERR_LAUNCH;
+  if (hipStreamSynchronize(st) != hipSuccess) return TMX_ERR_LAUNCH;
+  if (flag == 0) return TMX_OK;
+  if (hipMemsetAsync(word, 0, 4, st) != hipSuccess) return TMX_ERR_LAUNCH;
+  if (hipStreamSynchronize(st) != hipSuccess) return TMX_ERR_LAUNCH;
+  return TMX_ERR_DEVICE_WAIT;
 }
 
 // One decode step recorded into a HIP graph and replayed: the step index lives on the device,

@@ -805,8 +805,8 @@ struct GU8 {
 // hand-over is a write-through store (sc1) followed by a wait for its completion, the arrival counter
 // and the ready flag are device-scope atomics, and the readers load with sc1, so nothing depends on
 // the per-XCD L2 caches being written back or invalidated inside the kernel.  The main workgroups need
-// t only in their epilogue, long after the producers are done; their wait is bounded (a.sync[3] is set
-// and t taken as zero if the flag never comes).  The last reader puts the three counters back to zero,
+// t only in their epilogue, long after the producers are done; their wait is bounded (*a.sync_status is
+// set and t taken as zero if the flag never comes).  The last reader puts the three counters back to zero,
 // so the state is all-zero between launches (also under graph replay).
 __device__ __forceinline__ void sc1_store_b128(__amdgpu_buffer_rsrc_t r, u32x4_t v, int off) {
   __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, 0x10);
@@ -1069,7 +1069,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
         if (__hip_atomic_load(a.sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) { ok = 1; break; }
         __builtin_amdgcn_s_sleep(1);
       }
-      if (!ok) __hip_atomic_store(a.sync + 3, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (!ok && a.sync_status) __hip_atomic_store(a.sync_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_ready = ok;
     }
     __syncthreads();
@@ -1707,7 +1707,7 @@ size_t qlinear_gate_up_sync_bytes(int M, int K) {
 
 int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
-                           int F, int G, void* sync_ws) {
+                           int F, int G, void* sync_ws, uint32_t* status) {
   if (!x || !qw || !scales || !act) return TMX_ERR_ARG;
   if (M <= 0 || M > 128 || !four_wave_shape(K) || F % 64 || G % 64 || (G & (G - 1)) || K % G || ldx % 8)
     return TMX_ERR_SHAPE;
@@ -1743,6 +1743,7 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
       // that has no CU to run on
       const int mt = M <= 32 ? 1 : 2;
       a.sync = (uint32_t*)sync_ws;
+      a.sync_status = status;
       a.sync_part = (float*)((char*)sync_ws + 256);
       a.sync_t16 = (uint16_t*)((char*)sync_ws + 256 + (size_t)(K / 256) * mt * 4096);
       a.sync_blocks = mt == 1 ? K / 512 : K / 256;  // 8 / MT k-tiles per producer

@@ -35,6 +35,7 @@ struct QLinearArgs {
   // LoRA projection computed once per launch by extra workgroups and handed over through memory
   // (fused gate | up kernel): hand-over state {arrivals, ready, readers, timeout}, partial tiles, t
   uint32_t* sync;
+  uint32_t* sync_status;  // word set to 1 when a consumer's wait runs out (may be null)
   float* sync_part;
   uint16_t* sync_t16;
   int sync_blocks;
@@ -264,7 +265,7 @@ int qlinear_num_lora_splits(int K, int N);
 // leaves them so), or null: then every workgroup multiplies x by A itself
 int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
-                           int F, int G, void* sync_ws);
+                           int F, int G, void* sync_ws, uint32_t* status = nullptr);
 size_t qlinear_gate_up_sync_bytes(int M, int K);
 int zero_words(hipStream_t st, uint32_t* p, int n);  // p[0 .. n) = 0 by a small kernel
 // Many rows (M > 128), unsplit: y_bf16 = bf16(bf16(x . W) + bf16(bf16(t . B) ls)) in one pass, t = bf16(x . A)

@@ -220,7 +220,8 @@ class Sampler:
     ws_bytes = self._lib.tmx_decode_workspace_bytes(
         ctypes.byref(self._transformer.desc()), b * tokens_per_pass, self.cache_config.cache_size)
     if self._workspace is None or self._workspace.numel() < ws_bytes:
-      self._workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=self._transformer.device)
+      # zero-filled: the first 256 bytes hold the status word tmx_decode_status reads
+      self._workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=self._transformer.device)
     s = DecodeState()
     s.tokens_per_pass = tokens_per_pass
     s.batch, s.buf_len, s.cache_size = b, total, self.cache_config.cache_size
@@ -304,6 +305,13 @@ class Sampler:
             1 if sample else 0)
     _lib.check(rc, 'tmx_decode_steps_graph' if graph else 'tmx_decode_steps')
 
+  def check_device_status(self, st):
+    """Waits for the stream and raises if a bounded wait inside a kernel ran out since the last
+    check (tmx_decode_status); called before results are handed to the caller."""
+    cs = self._c_state(st)
+    rc = self._lib.tmx_decode_status(ctypes.byref(self._transformer.desc()), ctypes.byref(cs), _lib.stream())
+    _lib.check(rc, 'tmx_decode_status')
+
   def per_token_logps(self, prompt_tokens, completion_tokens, pad_id=None, temperature=1.0, token_mask=None):
     """Teacher-forced log-probabilities of the completion tokens, f32 [B, completion_len]:
     log_softmax(logits / temperature)[token] at every completion position given everything
@@ -339,6 +347,7 @@ class Sampler:
     st['sampling_mode'] = 'score'
     self.walk(st, p - 1)
     self.walk(st, t, sample=True)
+    self.check_device_status(st)
     return st['logprobs'][:, p:p + t].cpu().numpy()
 
   # -- the call ---------------------------------------------------------------
@@ -389,6 +398,7 @@ class Sampler:
           logits_steps.append(st['logits'].clone())
         if remaining > 0 and bool(st['done'].all().item()):
           break
+    self.check_device_status(st)
     token_buffers = st['token_buffer'].cpu().numpy()
     logprob_buffers = st['logprobs'].cpu().numpy() if return_logprobs else None
     if return_logits and logits_steps:
