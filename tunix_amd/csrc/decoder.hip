@@ -466,8 +466,9 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       }
       if (prof) TMX_TRY(TMX_K_EMPTY, empty_launch(st));
     }
-    if (sample && !nucleus && B > 128 && !s->logits_out && s->n_forbidden == 0 && D % 128 == 0) {
-      // many rows: the matrix-pipe-bound head kernel
+    if (sample && !nucleus && B > 64 && !s->logits_out && s->n_forbidden == 0 && D % 128 == 0) {
+      // more than 64 rows: the head in 256 x 256 blocks, one pass over the head matrix (the 64-row kernel
+      // would take one pass per 64 rows)
       HeadArgs a = {};
       a.x = w.xn;
       a.w = (const uint16_t*)m->head;

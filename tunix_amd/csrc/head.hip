@@ -397,12 +397,14 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
   const int target = score ? a.token_buffer[(size_t)(tok_l / tpp) * a.buf_len + min(*a.step + tok_l % tpp + 1, a.buf_len - 1)] : -1;
   float mx = kNegBig, se = 0.f;
   Best best = {-INFINITY, -INFINITY, 0x7FFFFFFF};
+  uint64_t packed = 0;  // sorting branch: the 16-bit keys of four consecutive vocabulary rows
+  const bool keys_out = sampling && a.sort_keys != nullptr && tok < a.M;
   // (unrolled by construction: a loop the compiler declines to unroll would index the accumulators
   // dynamically and move them to scratch memory)
   static_for<MT * 16>([&](auto ic) __attribute__((always_inline)) {
       constexpr int m = decltype(ic)::value / 16, r = decltype(ic)::value % 16;
       const int v = v0 + m * 32 + acc_row(r, lane);
-      if (v >= a.V) return;
+      if (v >= a.V) return;  // (V % 32 == 0 where keys are written: a group of four rows is in or out as one)
       const float logit = rbf(acc[m][r]);
       float z = logit, key = logit;
       if (score) {
@@ -410,9 +412,22 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
         key = (v == target) ? 0.f : -INFINITY;
       } else if (sampling) {
         z = logit / a.temperature;
-        uint32_t o0, o1;
-        threefry2x32(key0, key1, 0u, (uint32_t)tok_l * (uint32_t)a.V + (uint32_t)v, o0, o1);
-        key = z + gumbel_from_bits(o0 ^ o1);
+        if (a.sort_keys) {
+          // the same 16-bit descending key as head_kernel writes (selection happens in nucleus.hip)
+          if (keys_out) {
+            const uint32_t zb = __float_as_uint(logit + 0.0f) >> 16;
+            packed |= (uint64_t)((zb & 0x8000u) ? zb : (~zb & 0x7FFFu)) << (16 * (r & 3));
+            if constexpr ((r & 3) == 3) {
+              *reinterpret_cast<uint64_t*>(a.sort_keys + (size_t)tok * a.V + v - 3) = packed;
+              packed = 0;
+            }
+          }
+          key = z;
+        } else {
+          uint32_t o0, o1;
+          threefry2x32(key0, key1, 0u, (uint32_t)tok_l * (uint32_t)a.V + (uint32_t)v, o0, o1);
+          key = z + gumbel_from_bits(o0 ^ o1);
+        }
       }
       if (z > mx) {
         se = se * expf(mx - z) + 1.f;
@@ -452,9 +467,14 @@ static int launch_head_wide(hipStream_t st, const HeadArgs& a, int tok_blocks, i
   return TMX_OK;
 }
 
-int head_wide(hipStream_t st, HeadArgs a) {
-  if (a.D % 128 || a.M <= 0 || (size_t)a.M * a.D * 2 >= (1u << 31) || (size_t)256 * a.D * 2 >= (1u << 31))
-    return TMX_ERR_SHAPE;
+bool head_wide_ok(const HeadArgs& a) {
+  return a.D % 128 == 0 && a.M > 0 && (size_t)a.M * a.D * 2 < (1u << 31) && (size_t)256 * a.D * 2 < (1u << 31) &&
+         a.n_forbidden == 0 && !a.logits_out;
+}
+
+// The wide kernel alone: partials (and, in the sorting branch, keys) of every row; sets a.nwg.
+int head_wide_logits(hipStream_t st, HeadArgs& a) {
+  if (!head_wide_ok(a)) return TMX_ERR_SHAPE;
   const int tok_blocks = (a.M + 255) / 256, voc_blocks = (a.V + HW::ROWS - 1) / HW::ROWS;
   a.nwg = voc_blocks;
   a.row_base = 0;
@@ -463,7 +483,11 @@ int head_wide(hipStream_t st, HeadArgs a) {
   else if (a.mode == TMX_SAMPLE_TOP_P) lrc = launch_head_wide<TMX_SAMPLE_TOP_P>(st, a, tok_blocks, voc_blocks);
   else lrc = launch_head_wide<TMX_SAMPLE_GREEDY>(st, a, tok_blocks, voc_blocks);
   if (lrc != TMX_OK) return lrc;
-  int rc = check_launch();
+  return check_launch();
+}
+
+int head_wide(hipStream_t st, HeadArgs a) {
+  int rc = head_wide_logits(st, a);
   if (rc != TMX_OK) return rc;
   hipLaunchKernelGGL(head_finalize_kernel, dim3(a.M), dim3(256), 0, st, a);
   return check_launch();

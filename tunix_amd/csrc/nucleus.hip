@@ -435,7 +435,8 @@ int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void
   if (attr != hipSuccess || attr2 != hipSuccess || attr3 != hipSuccess) return TMX_ERR_LAUNCH;
   a.mode = TMX_SAMPLE_TOP_P;
   a.sort_keys = c.keys;
-  int rc = head_logits(st, a);
+  // more than 64 rows: one pass over the head matrix in 256 x 256 blocks instead of one per 64 rows
+  int rc = (a.M > 64 && head_wide_ok(a)) ? head_wide_logits(st, a) : head_logits(st, a);
   if (rc != TMX_OK) return rc;
   NucleusArgs n = {};
   n.keys = c.keys; n.ent = c.ent; n.tot = c.tot; n.pbest = c.pbest;

@@ -255,6 +255,8 @@ int head_sample(hipStream_t st, HeadArgs a);
 // any number of rows in 256 x 256 blocks (greedy, sampling without the sorting branch, scoring); needs
 // D % 128 == 0, no forbidden ids, no logits output; part_f / part_i sized [M][ceil(V / 256)]
 int head_wide(hipStream_t st, HeadArgs a);
+bool head_wide_ok(const HeadArgs& a);
+int head_wide_logits(hipStream_t st, HeadArgs& a);  // the wide kernel without the finalize launch
 int head_logits(hipStream_t st, HeadArgs& a);  // the vocabulary kernel alone; fills a.nwg
 int head_sample_nucleus(hipStream_t st, HeadArgs a, float top_p, int top_k, void* ws, size_t ws_bytes);
 size_t nucleus_bytes(int M, int V);
