@@ -361,12 +361,14 @@ def test_moe_decoder_matches_oracle():
   _compare_greedy(out, ref, 4, min_checked=20, lp_extra=2.0 ** -7)
 
 
-@pytest.mark.parametrize('nseq', [4, 150])
-def test_graph_replay_matches_plain_launches_on_every_replay(nseq):
+@pytest.mark.parametrize('nseq,top_p', [(4, 1.0), (150, 1.0), (6, 0.8), (70, 0.9)])
+def test_graph_replay_matches_plain_launches_on_every_replay(nseq, top_p):
   """tmx_decode_steps_graph against tmx_decode_steps: several graph calls in a row, with the
   program's own eager work (a plain step, host reads) and synchronisation between them; every
-  call's tokens, logprobs, KV cache and step counter equal the plain launches'.  150 sequences:
-  the launches of the many-rows kernels are recorded."""
+  call's tokens, logprobs, KV cache and step counter equal the plain launches'.  4 sequences: the
+  small-batch launches; 150: the many-rows kernels; top_p < 1: the selection launches of the
+  top-p branch (6 sequences behind the 64-row head and the gate|up hand-over, 70 behind the head in
+  256 x 256 blocks) are recorded and replayed."""
   cfg = C.TOY
   _, model = _pair(cfg, seed=17, targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
   rng = np.random.default_rng(2)
@@ -374,7 +376,7 @@ def test_graph_replay_matches_plain_launches_on_every_replay(nseq):
   def run(graph):
     s = _sampler(model, cfg, 64)
     s.eos_ids = np.array([-1])
-    st = s.init_sample_state(ids, 64, False, None, 0.9, 1.0, None, 5, include_logprobs=True,
+    st = s.init_sample_state(ids, 64, False, None, 0.9, top_p, None, 5, include_logprobs=True,
                              prompt_lengths=np.full(nseq, 8))
     snaps = []
     s.run_steps(st, 7, sample=False, graph=graph)
