@@ -679,7 +679,7 @@ def test_moe_experts_match_oracle(B, D, F, E, k, group):
     (1, 2048, 3072, 64, 16, 'norm'), (1, 2048, 2048, 64, 16, 'residual'), (1, 2048, 1024, 64, 16, 'swiglu'),
     (1, 8192, 2048, 64, 16, 'residual'), (4, 256, 96, 64, 8, 'norm'), (3, 512, 256, 128, 0, 'plain'),
     (2, 1024, 256, 64, 32, 'residual'), (4, 512, 128, 64, 4, 'swiglu'), (1, 320, 64, 64, 0, 'swiglu'),
-    (1, 2048, 3072, 64, 0, 'norm_qwen')])
+    (1, 2048, 3072, 64, 0, 'norm_qwen'), (1, 2048, 16384, 64, 16, 'swiglu'), (4, 2048, 16384, 64, 16, 'swiglu')])
 def test_small_linear_matches_oracle(M, K, N, group, r, mode):
   T = G.Keep()
   rng = np.random.default_rng(M * 13 + K + N)
@@ -726,7 +726,9 @@ def test_small_linear_matches_oracle(M, K, N, group, r, mode):
   got = G.host(y)
   if swiglu:
     # a last-bit flip of gate or up (f32 summation order) moves the product by about an ulp of it
-    G.assert_bf16_close(got, want, ulps=2.0, extra=1e-6 + 2.0 * G.ulp_bf16(want), min_exact=0.97, what=f'small swiglu {K}x{N}')
+    # (gate and up both flipping on one element is rare: a couple of elements in 32768 may reach three bounds)
+    G.assert_bf16_close(got, want, ulps=2.0, extra=1e-6 + 2.0 * G.ulp_bf16(want), min_exact=0.97, what=f'small swiglu {K}x{N}',
+                        stragglers=2 if want.size > 8192 else 0)
   else:
     extra = (G.ulp_bf16(base) + G.ulp_bf16(out)) if (r or mode == 'residual') else 0.0
     if r:
