@@ -265,3 +265,49 @@ def test_model_from_state_tree_flattens_before_it_builds(monkeypatch):
   assert QLoRAModel.from_state_tree(ModelConfig.toy(), tree, group=64, lora_alpha=8.0, device='cpu') == 'built'
   assert set(seen['state']) == {'layers.0.attn.q_proj.w', 'layers.0.attn.q_proj.w_lora_a', 'embedder.input_embedding'}
   assert tuple(seen['state']['layers.0.attn.q_proj.w'].shape) == (4, 2, 3) and seen['kw']['lora_alpha'] == 8.0
+
+
+def test_rollout_takes_the_actor_forms_the_cluster_hands_over(monkeypatch):
+  """TmxRollout(rollout_actor=...): a (reference config, state tree) pair is converted with the
+  reference's field names (llama3/model.py:85-101, qwen3/model.py:160-185); an nnx module without
+  flax importable and anything else raise TypeError (no GPU: the quantising constructor is stubbed)."""
+  import dataclasses as dc
+  from tunix_amd.model import QLoRAModel
+  from tunix_amd.rollout import TmxRollout
+
+  @dc.dataclass
+  class RefLlama:  # the reference's Llama3 ModelConfig, fields only
+    num_layers: int = 2
+    vocab_size: int = 1024
+    embed_dim: int = 256
+    hidden_dim: int = 1024
+    num_heads: int = 4
+    head_dim: int = 64
+    num_kv_heads: int = 4
+    rope_theta: int = 10_000
+    norm_eps: float = 1e-5
+    weight_tying: bool = True
+
+  @dc.dataclass
+  class RefQwen(RefLlama):
+    use_tied_embedding: bool = False
+    num_experts: int = 8
+    num_experts_per_tok: int = 2
+
+  c = ModelConfig.from_reference(RefLlama())
+  assert (c.family, c.num_layers, c.vocab_size, c.head_dim, c.weight_tying, c.num_experts) == ('llama3', 2, 1024, 64, True, None)
+  q = ModelConfig.from_reference(RefQwen(weight_tying=False))
+  assert (q.family, q.weight_tying, q.num_experts, q.num_experts_per_tok) == ('qwen3', False, 8, 2)
+  seen = {}
+  monkeypatch.setattr(QLoRAModel, 'from_state_tree',
+                      classmethod(lambda cls, cfg, tree, **kw: seen.update(cfg=cfg, tree=tree, kw=kw) or 'policy'))
+  tree = {'layers': {0: {}}}
+  assert TmxRollout._as_policy((RefLlama(), tree), 128, 32.0, 7.5) == 'policy'
+  assert seen['cfg'].family == 'llama3' and seen['tree'] is tree and seen['kw'] == {'group': 128, 'lora_alpha': 32.0, 'bound': 7.5}
+
+  class Module:  # stands for an nnx module: has .config, its state needs flax
+    config = RefLlama()
+  with pytest.raises(TypeError, match='flax is not importable'):
+    TmxRollout._as_policy(Module(), 64, None, 7.5)
+  with pytest.raises(TypeError, match='expected a QLoRAModel'):
+    TmxRollout._as_policy(object(), 64, None, 7.5)

@@ -38,6 +38,21 @@ class ModelConfig:
   num_experts_per_tok: Optional[int] = None
 
   @classmethod
+  def from_reference(cls, cfg, family=None):
+    """From one of the reference's own ModelConfig objects (llama3/model.py:85-101,
+    qwen3/model.py:160-185), read by attribute name; `family` is taken from the defining module or
+    from the Qwen3-only fields when not given."""
+    if family is None:
+      mod = type(cfg).__module__ or ''
+      family = 'qwen3' if ('qwen3' in mod or hasattr(cfg, 'use_tied_embedding')) else 'llama3'
+    if family not in ('llama3', 'qwen3'):
+      raise ValueError(f'unknown model family {family!r}')
+    tied = bool(getattr(cfg, 'weight_tying', False) or getattr(cfg, 'use_tied_embedding', False))
+    return cls(family, int(cfg.num_layers), int(cfg.vocab_size), int(cfg.embed_dim), int(cfg.hidden_dim),
+               int(cfg.num_heads), int(cfg.head_dim), int(cfg.num_kv_heads), float(cfg.rope_theta),
+               float(cfg.norm_eps), tied, getattr(cfg, 'num_experts', None), getattr(cfg, 'num_experts_per_tok', None))
+
+  @classmethod
   def llama3p2_1b(cls):
     return cls('llama3', 16, 128256, 2048, 8192, 32, 64, 8, 500_000, 1e-5, True)
 

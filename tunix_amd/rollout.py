@@ -43,15 +43,42 @@ class TmxRollout(BaseRollout):
 
   Accepts both construction styles of the reference: positional
   (model, tokenizer, cache_config) like VanillaRollout, or the engine keywords
-  (rollout_actor, tokenizer, mesh, rollout_config) of a user-defined engine.
+  (rollout_actor, tokenizer, mesh, rollout_config) of a user-defined engine
+  (tunix/rl/rl_cluster.py:388-410 hands over the nnx actor itself).  The actor may be a
+  QLoRAModel, a (reference ModelConfig, state tree) pair, or the reference's LoRA-wrapped nnx
+  module (needs flax importable to read its state); the latter two are quantised here, once,
+  with `group` / `lora_alpha` / `quant_bound` (bind them with functools.partial).
   """
 
+  @staticmethod
+  def _as_policy(actor, group, lora_alpha, quant_bound):
+    from tunix_amd.model import ModelConfig, QLoRAModel
+    if isinstance(actor, QLoRAModel) or isinstance(getattr(actor, 'config', None), ModelConfig):
+      return actor  # already a policy of this package (its config is this package's ModelConfig)
+    if isinstance(actor, tuple) and len(actor) == 2:
+      cfg, tree = actor
+    elif hasattr(actor, 'config'):
+      try:
+        from flax import nnx
+      except ImportError as e:
+        raise TypeError('rollout_actor is an nnx module but flax is not importable to read its state: pass a '
+                        'QLoRAModel (QLoRAModel.from_state_tree) or a (config, state tree) pair') from e
+      cfg, tree = actor.config, nnx.state(actor)
+    else:
+      raise TypeError(f'rollout_actor of type {type(actor).__name__}: expected a QLoRAModel, a (config, state tree) '
+                      'pair or an nnx module with .config')
+    if not isinstance(cfg, ModelConfig):
+      cfg = ModelConfig.from_reference(cfg)
+    return QLoRAModel.from_state_tree(cfg, tree, group=group, lora_alpha=0.0 if lora_alpha is None else lora_alpha,
+                                      bound=quant_bound)
+
   def __init__(self, model=None, tokenizer=None, cache_config_or_size=None, *, rollout_actor=None,
-               mesh=None, rollout_config: RolloutConfig = None):
+               mesh=None, rollout_config: RolloutConfig = None, group=64, lora_alpha=None, quant_bound=7.5):
     del mesh  # one GPU: nothing to shard
     actor = model if model is not None else rollout_actor
     if actor is None or tokenizer is None:
       raise ValueError('a model (rollout_actor) and a tokenizer are required')
+    actor = self._as_policy(actor, group, lora_alpha, quant_bound)
     if cache_config_or_size is None:
       if rollout_config is None:
         raise ValueError('either cache_config_or_size or rollout_config is required')
