@@ -34,6 +34,20 @@ def test_library_exports_every_declared_symbol():
   assert set(syms) <= bound, sorted(set(syms) - bound)
 
 
+def test_header_is_plain_c_and_cxx():
+  """include/tmx.h is the boundary a foreign-function binding reads: it must compile as C99 and as C++
+  on its own (no torch, HIP or C++-only types in any signature)."""
+  import shutil
+  import subprocess
+  hdr = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), 'include', 'tmx.h')
+  for cc, lang, std in (('gcc', 'c', '-std=c99'), ('g++', 'c++', '-std=c++11')):
+    if shutil.which(cc) is None:
+      pytest.skip(f'{cc} is not installed')
+    res = subprocess.run([cc, std, '-Wall', '-Wextra', '-Werror', '-pedantic', '-fsyntax-only', '-x', lang, hdr],
+                         capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+
+
 def test_status_strings_and_version():
   lib = _lib.lib()
   assert lib.tmx_abi_version() == 4
