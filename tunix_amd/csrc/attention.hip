@@ -23,7 +23,7 @@ template <int G>
 struct AttnWaves { static constexpr int value = G > 4 ? 2 : 4; };
 
 template <int H, int G>
-__global__ __launch_bounds__(AttnWaves<G>::value * 64) void gqa_decode_kernel(AttnArgs a) {
+__global__ __launch_bounds__(AttnWaves<G>::value * 64, 4) void gqa_decode_kernel(AttnArgs a) {
   constexpr int NW = AttnWaves<G>::value;
   constexpr int LPP = H / 8;     // lanes per position row
   constexpr int PPW = 64 / LPP;  // positions per wave-wide load
