@@ -108,6 +108,21 @@ int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight, co
                             const void* lora_a_t, float* y_part, float* t_part, int M, int K, int N,
                             int G, int r_pad, int nsplit);
 
+/* tmx_qlora_linear_planes whose launch also finishes the LoRA product: once every slice of x . A is
+ * there, the LoRA workgroups of the launch add the planes in slice order, round to bf16 and write
+ * delta[M, N] = bf16(bf16(t . B) * lora_scale) (bf16), the term the consumer adds to the rounded sum of the
+ * y planes (column n below seg_end0 uses t columns 0..r-1, below seg_end1 r..2r-1, else 2r..3r-1: the
+ * fused q | k | v layout; pass N, N for a single matrix).  This is what the decode step does for
+ * projections whose K-slices are long enough to hide it (slices of at least 2048 rows of W, at most two
+ * 32-column tiles per LoRA wave): tmx_qlora_linear_delta_workspace_bytes returns 0 for every other shape
+ * and the call TMX_ERR_UNSUPPORTED.  workspace: that many bytes (cleared by the call: one small launch).
+ * Up to 128 rows, r <= 64.  No counterpart in the reference beyond the LoRA arithmetic itself. */
+size_t tmx_qlora_linear_delta_workspace_bytes(int M, int K, int N, int r, int r_pad, int nsplit);
+int tmx_qlora_linear_planes_delta(void* stream, const void* x, const void* qweight, const void* scales,
+                                  const void* lora_a_t, const void* lora_b, float* y_part, float* t_part,
+                                  void* delta, void* workspace, int M, int K, int N, int G, int r, int r_pad,
+                                  float lora_scale, int seg_end0, int seg_end1, int nsplit);
+
 /* One projection of the single-sequence regime (1..4 rows) in ONE launch: optional RMSNorm of
  * x in the prologue (norm_w != NULL; family as tmx_rmsnorm), the int4 product, the LoRA delta
  * computed inside (t = x . A by every workgroup), then either nothing, the residual add

@@ -673,6 +673,68 @@ def test_moe_experts_match_oracle(B, D, F, E, k, group):
   assert not np.isin(idx, E - 1).any()
 
 
+# ---- LoRA delta finished by the projection's own launch ----------------------------------------------
+
+@pytest.mark.parametrize('M,K,widths,group,r,nsplit', [
+    (64, 14336, (4096,), 64, 16, 7),        # the 8B down projection
+    (8, 8192, (2048,), 64, 8, 4),           # rank 8: half of the 16-wide rank step is masked
+    (32, 8192, (4096,), 128, 12, 2),        # rank not a multiple of 8: the element-wise fragment path
+    (128, 12288, (4096,), 128, 32, 4),      # 128 rows, two rank steps
+    (16, 8192, (2048, 512, 512), 64, 16, 2),  # three fused matrices (q | k | v): t columns by segment
+])
+def test_projection_writes_the_lora_delta(M, K, widths, group, r, nsplit):
+  """tmx_qlora_linear_planes_delta: the y planes add up to x . W as before, and delta equals
+  bf16(bf16(t . B) * s) with t = bf16(x . A) per fused matrix (tunix's qwix-wrapped Einsum, SURVEY a16:
+  (x . A) . B * alpha / rank), twice in a row on one workspace (its counters must be back at zero)."""
+  T = G.Keep()
+  lib = _lib.lib()
+  rng = np.random.default_rng(M + K + r)
+  N = sum(widths)
+  x = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+  ws = [bf16_round(rng.standard_normal((K, n)).astype(np.float32) * 0.02) for n in widths]
+  As = [bf16_round(rng.standard_normal((K, r)).astype(np.float32) * 0.05) for _ in widths]
+  Bs = [bf16_round(rng.standard_normal((r, n)).astype(np.float32) * 0.05) for n in widths]
+  ls = 2.0
+  pl = quant.PackedLinear.from_dense([torch.from_numpy(w) for w in ws], group, G.DEV,
+                                     [(torch.from_numpy(a), torch.from_numpy(b)) for a, b in zip(As, Bs)], ls)
+  nb = lib.tmx_qlora_linear_delta_workspace_bytes(M, K, N, r, pl.r_pad, nsplit)
+  assert nb > 0
+  nls = lib.tmx_qlora_linear_num_lora_splits(K, N)
+  wsb = torch.empty(nb, dtype=torch.uint8, device=G.DEV)
+  yp = torch.full((nsplit, M, N), float('nan'), dtype=torch.float32, device=G.DEV)
+  tp = torch.full((nls, M, 128), float('nan'), dtype=torch.float32, device=G.DEV)
+  ends = list(np.cumsum(widths))
+  e0, e1 = (ends[0], ends[1]) if len(widths) == 3 else (N, N)
+  outs = []
+  for _ in range(2):
+    d = torch.full((M, N), float('nan'), dtype=torch.bfloat16, device=G.DEV)
+    G.call('tmx_qlora_linear_planes_delta', S(), T.bf(x), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t), G.p(pl.lora_b),
+           G.p(yp), G.p(tp), G.p(d), G.p(wsb), M, K, N, group, r, pl.r_pad, ls, int(e0), int(e1), nsplit)
+    G.sync()
+    outs.append(G.host(d))
+  np.testing.assert_array_equal(outs[0], outs[1])
+  assert int(wsb[:16].view(torch.int32).abs().sum().item()) == 0
+  got = outs[1]
+  want = np.concatenate([bf16_round(bf16_round(bf16_round(x @ a) @ b) * ls) for a, b in zip(As, Bs)], axis=1)
+  # a last-bit flip of a t element (f32 summation order of x . A) moves the product by ulp(t) |B|
+  tt = [bf16_round(x @ a) for a in As]
+  slack = np.concatenate([(G.ulp_bf16(t) @ np.abs(b)) * ls for t, b in zip(tt, Bs)], axis=1)
+  G.assert_bf16_close(got, want, ulps=1.0, extra=slack + 2.0 ** -22 * np.abs(want), min_exact=0.9, what=f'delta {M}x{K}x{N} r{r}')
+  # the planes still add up to the base product
+  qs = [int4.quantize(w, group) for w in ws]
+  base = np.concatenate([x @ L.Linear(q=q, scale=sc, group=group).weight() for q, sc in qs], axis=1)
+  ysum = yp.sum(0).cpu().numpy()
+  np.testing.assert_allclose(ysum, base, rtol=2e-3, atol=2e-3 * np.abs(base).max())
+
+
+def test_projection_delta_only_where_it_hides():
+  lib = _lib.lib()
+  assert lib.tmx_qlora_linear_delta_workspace_bytes(64, 14336, 4096, 16, 32, 7) > 0
+  assert lib.tmx_qlora_linear_delta_workspace_bytes(64, 4096, 4096, 16, 32, 4) == 0   # 4-step slices: the stage would stick out
+  assert lib.tmx_qlora_linear_delta_workspace_bytes(64, 4096, 28672, 16, 32, 1) == 0  # too many column tiles per LoRA wave
+  assert lib.tmx_qlora_linear_delta_workspace_bytes(256, 14336, 4096, 16, 32, 7) == 0  # more than 128 rows
+
+
 # ---- single-sequence regime: norm | projection | LoRA | residual / SwiGLU in one launch -----------
 
 @pytest.mark.parametrize('M,K,N,group,r,mode', [

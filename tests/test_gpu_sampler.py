@@ -66,6 +66,25 @@ def test_toy_config_greedy_matches_oracle():
   _compare_greedy(out, ref, 4, 40)
 
 
+def test_wide_layer_with_the_projection_side_lora_delta_matches_oracle():
+  """One layer at the 8B width (d 4096, SwiGLU 14336, 32 / 8 heads of 128), LoRA r16 on every projection,
+  6 sequences: the down projection is long enough (7 K-slices of 2048) for its own launch to finish the
+  LoRA product, and the row kernel behind it adds that delta instead of multiplying by B.  Greedy tokens
+  and log-probs against the oracle, as for the toy configuration."""
+  from tunix_amd import _lib
+  cfg = OM.Config('llama3', 1, 512, 4096, 14336, 32, 128, 8, norm_eps=1e-5)
+  assert _lib.lib().tmx_qlora_linear_delta_workspace_bytes(6, 14336, 4096, 16, 32, _lib.lib().tmx_qlora_linear_num_splits(6, 14336, 4096)) > 0
+  oracle, model = _pair(cfg, seed=21, rank=16, alpha=32.0,
+                        targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
+  rng = np.random.default_rng(5)
+  prompts = [rng.integers(3, cfg.vocab_size, 5) for _ in range(6)]
+  ref = OSAM.generate(oracle, cfg, prompts, 5, 16, eos_ids=(-1,))
+  out = _sampler(model, cfg, 16)(prompt_token_ids=prompts, max_generation_steps=5, return_logprobs=True, eos_tokens=[-1])
+  # 4096-wide hidden states against a 0.02-std head give logits of a few units: one bf16 ulp of the chosen logit
+  # (2^-6 .. 2^-5 there, against 2^-8 on the toy width) is the resolution of the log-prob itself
+  _compare_greedy(out, ref, 6, 12, lp_extra=2.0 ** -5)
+
+
 def test_left_padded_ragged_prompts_and_all_lora_targets():
   cfg = OM.Config('llama3', 2, 512, 256, 512, 8, 64, 2, norm_eps=1e-5)  # GQA group of 4
   oracle, model = _pair(cfg, seed=3, rank=16, alpha=32.0,

@@ -18,6 +18,7 @@ SIGNATURES = {
     'tmx_int4_dequant': [vp, vp, vp, vp, ci, ci, ci],
     'tmx_qlora_linear': [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
     'tmx_qlora_linear_noalloc': [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf],
+    'tmx_qlora_linear_planes_delta': [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf, ci, ci, ci],
     'tmx_small_linear': [vp, vp, vp, cf, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cf, ci],
     'tmx_qlora_linear_num_splits': [ci, ci, ci],
     'tmx_qlora_linear_num_lora_splits': [ci, ci],
@@ -48,6 +49,7 @@ SIZE_FUNCS = {
     'tmx_qlora_linear_noalloc_max_bytes': [],
     'tmx_head_sample_workspace_bytes': [ci, ci],
     'tmx_nucleus_workspace_bytes': [ci, ci],
+    'tmx_qlora_linear_delta_workspace_bytes': [ci, ci, ci, ci, ci, ci],
     'tmx_decode_workspace_bytes': [vp, ci, ci],
 }
 

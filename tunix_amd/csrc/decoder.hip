@@ -17,6 +17,8 @@ namespace tmx {
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Workspace {
+  uint16_t* delta;   // LoRA delta of a split projection, made by its LoRA blocks (up to 128 rows)
+  void* dsync;       // their hand-over area
   uint32_t* status;  // first 256 bytes, the same place for every batch size: word 0 is set when a bounded wait inside a kernel runs out
   uint16_t *x, *xn, *q, *attn, *act, *y16;
   float *y_part, *t_part, *rope_tab;
@@ -102,6 +104,10 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   w.y_part = (float*)take((size_t)B * ypart * 4);
   w.t_part = (float*)take((size_t)TMX_MAX_LORA_SPLITS * B * TMX_MAX_RPAD * 4);
   w.t16 = (uint16_t*)take(B > 128 ? (size_t)B * TMX_MAX_RPAD * 2 : 0);
+  {
+    w.delta = (uint16_t*)take(B <= 128 ? (size_t)B * D * 2 : 0);
+    w.dsync = take(B <= 128 ? qlinear_delta_sync_bytes(B, TMX_MAX_RPAD) : 0);
+  }
   w.gu_sync = take(B <= kFusedGateUpMaxRows && m->num_experts == 0 && D % 256 == 0 ? qlinear_gate_up_sync_bytes(B, (int)D) : 0);
   const bool small = B <= kSmallBatchMaxRows && m->num_experts == 0;
   w.sb_tparts = (float*)take(small ? (F / 32 + 1) * (size_t)B * 32 * 4 : 0);
@@ -210,6 +216,23 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     }
     return li;
   };
+  // Up to 128 rows, o and down projections of the direct-to-LDS kernel whose K-slices are long enough to hide
+  // it: the LoRA blocks of the launch also make delta = bf16(bf16(t . B) * ls), so the row kernel behind adds one
+  // bf16 row instead of multiplying by B (every row re-read all of B there).
+  auto delta_of = [&](const tmx_qlinear_desc& l, int nsplit, int e0, int e1, LoraDelta& ld) {
+    if (!l.lora_a_t || !w.delta || !w.dsync || e0 % 32 || e1 % 32) return false;
+    if (!qlinear_delta_ok(B, l.K, l.N, l.r_pad, l.rank, nsplit)) return false;
+    ld = LoraDelta();
+    ld.delta = w.delta;
+    ld.lora_b = (const uint16_t*)l.lora_b; ld.r = l.rank; ld.ls = l.lora_scale;
+    ld.seg_end[0] = e0; ld.seg_end[1] = e1; ld.seg_end[2] = l.N;
+    ld.sync_ws = w.dsync; ld.status = w.status;
+    return true;
+  };
+  if (w.dsync && n_steps > 0) {  // the hand-over words start at zero (the kernel leaves them so)
+    rc = zero_words(st, (uint32_t*)w.dsync, 64);
+    if (rc != TMX_OK) return rc;
+  }
   // Many rows (B > 128): projection + LoRA in one pass into w.y16 where the shape allows it (unsplit,
   // rank % 8 == 0); returns TMX_ERR_UNSUPPORTED (nothing launched) when the caller must take the planes path.
   auto wide_linear = [&](const void* x, int ldx, const tmx_qlinear_desc& l, int e0, int e1) {
@@ -318,6 +341,8 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       uint16_t* kc = (uint16_t*)s->kv_cache + (size_t)(2 * i) * kv_elems;
       uint16_t* vc = kc + kv_elems;
       bool fused;  // this projection ran with LoRA in its epilogue: the consumer reads bf16, no LoRA left
+      LoraDelta ld;
+      bool with_delta = false;  // the projection's LoRA blocks made the delta: the consumer adds it
       {
         if (prof) prof->before(TMX_K_QKV, st);
         rc = wide_linear(w.xn, D, l.qkv, NH, NH + Kh * H);
@@ -359,9 +384,11 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         if (prof) prof->before(TMX_K_O, st);
         rc = wide_linear(w.attn, NH, l.o, D, D);
         fused = rc != TMX_ERR_UNSUPPORTED;
-        if (!fused)
+        if (!fused) {
+          with_delta = delta_of(l.o, sp.o, D, D, ld);
           rc = qlinear_base(st, w.attn, NH, l.o.qweight, l.o.scales, l.o.lora_a_t, nullptr, w.y_part, w.t_part,
-                            TMX_MAX_RPAD, B, NH, D, l.o.G, l.o.r_pad, sp.o);
+                            TMX_MAX_RPAD, B, NH, D, l.o.G, l.o.r_pad, sp.o, with_delta ? &ld : nullptr);
+        }
         if (prof) prof->after(TMX_K_O, st);
         if (rc != TMX_OK) return rc;
       }
@@ -372,7 +399,8 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         } else {
           a.y_part = w.y_part;
           a.nsplit = sp.o;
-          a.lora = lora_of(l.o, sp.o);
+          if (with_delta) a.delta = w.delta;
+          else a.lora = lora_of(l.o, sp.o);
         }
         a.residual = w.x; a.x_out = w.x;
         a.norm_w = (const uint16_t*)l.norm2_w; a.xn_out = w.xn;
@@ -442,9 +470,11 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
           if (prof) prof->before(TMX_K_DOWN, st);
           rc = wide_linear(w.act, F, l.down, D, D);
           fused = rc != TMX_ERR_UNSUPPORTED;
-          if (!fused)
+          if (!fused) {
+            with_delta = delta_of(l.down, sp.down, D, D, ld);
             rc = qlinear_base(st, w.act, F, l.down.qweight, l.down.scales, l.down.lora_a_t, nullptr, w.y_part,
-                              w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G, l.down.r_pad, sp.down);
+                              w.t_part, TMX_MAX_RPAD, B, F, D, l.down.G, l.down.r_pad, sp.down, with_delta ? &ld : nullptr);
+          }
           if (prof) prof->after(TMX_K_DOWN, st);
           if (rc != TMX_OK) return rc;
         }
@@ -455,7 +485,8 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
           } else {
             a.y_part = w.y_part;
             a.nsplit = sp.down;
-            a.lora = lora_of(l.down, sp.down);
+            if (with_delta) a.delta = w.delta;
+            else a.lora = lora_of(l.down, sp.down);
           }
           a.residual = w.x; a.x_out = w.x;
           a.norm_w = (const uint16_t*)(i + 1 < m->num_layers ? m->layers[i + 1].norm1_w : m->final_norm_w);

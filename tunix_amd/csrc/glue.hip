@@ -247,11 +247,18 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
         for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e]);
         if (a.residual) unpack8(*reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0), res8[i]);
       } else {
-        // the residual is requested before the planes are waited for
-        uint4 r4 = {0, 0, 0, 0};
+        // the residual (and the LoRA delta, when the projection made it) is requested before the planes are waited for
+        uint4 r4 = {0, 0, 0, 0}, d4 = {0, 0, 0, 0};
         if (a.residual) r4 = *reinterpret_cast<const uint4*>(a.residual + (size_t)m * a.D + n0);
+        if (a.delta) d4 = *reinterpret_cast<const uint4*>(a.delta + (size_t)m * a.D + n0);
         load_base8(a.y_bf16, a.y_part, a.nsplit, m, M, a.D, n0, v[i]);
         if (a.residual) unpack8(r4, res8[i]);
+        if (a.delta) {  // bf16(base + delta), delta = bf16(bf16(t . B) * ls)
+          float d8[8];
+          unpack8(d4, d8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e] + d8[e]);
+        }
       }
     }
   }

@@ -1192,6 +1192,150 @@ struct KD {
   static constexpr size_t lds(int MT) { return (size_t)2 * MT * 32 * XS * 2; }
 };
 
+// LoRA delta by the LoRA blocks of a split projection.  Every LoRA block that holds k-tiles has stored
+// its plane of t = x . A with write-through stores and counts itself in (stores complete before the
+// counter moves).  Then ALL LoRA blocks of the launch (also those whose slice is empty) wait until every
+// slice has arrived, a bounded number of polls; each adds the planes in slice order (loads past its L2),
+// rounds to bf16, and takes its share of the column tiles of delta = bf16(bf16(t . B) * ls): t rows are
+// the MFMA A operand, B columns the B operand, the rank in steps of 16 with zeros past it.  The B
+// fragments of a wave's first tiles are requested before the wait.  The main blocks never wait for any
+// of this, and the LoRA blocks' slices are short, so the stage runs while the main blocks still
+// multiply.  The last block to finish puts the two counters back to zero.
+template <int MT>
+__device__ __forceinline__ void lora_delta_stage(const QLinearArgs& a, uint16_t* smem, const bool holds_slice) {
+  __shared__ uint32_t s_flag;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, nl = lane & 31;
+  const int L = a.lora_blocks_per_split * a.nsplit;
+  const int me = ((int)blockIdx.x - a.n_main_blocks) + a.lora_blocks_per_split * (int)blockIdx.y;
+  const int rows = a.M < MT * 32 ? a.M : MT * 32;
+  const __amdgpu_buffer_rsrc_t rp = make_rsrc(a.t_part, 0x7FFFFFFFu);
+  if (holds_slice) {
+    __builtin_amdgcn_s_waitcnt(0);  // this block's plane is in memory
+    __syncthreads();
+    if (tid == 0) __hip_atomic_fetch_add(a.sync + 0, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // B fragments (rank step 0) of this wave's first tiles: they do not depend on t
+  constexpr int PT = 2;  // host: at most two tiles per wave
+  const int ntiles = a.N >> 5, ksteps = (a.lora_r + 15) >> 4, tstride = L * 8;
+  const int tile0 = me * 8 + wave;
+  bf16x8_t tb0[PT];
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int tile = tile0 + i * tstride;
+    uint16_t bz[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = h * 8 + j;
+      bz[j] = (tile < ntiles && k < a.lora_r) ? a.lora_b[(size_t)k * a.N + tile * 32 + nl] : (uint16_t)0;
+    }
+    __builtin_memcpy(&tb0[i], bz, 16);
+  }
+  if (tid == 0) {
+    uint32_t ok = 0;
+    for (int spin = 0; spin < (1 << 20); ++spin) {
+      if (__hip_atomic_load(a.sync + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)a.n_lora_slices) { ok = 1; break; }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (!ok && a.sync_status) __hip_atomic_store(a.sync_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_flag = ok;
+  }
+  __syncthreads();
+  const bool ready = s_flag != 0;  // false: t is taken as zero (the status word says so)
+  // t = bf16(sum of the planes in slice order) into LDS (the slab area is free), bf16 [MT * 32][Rpad];
+  // a thread takes four adjacent columns, up to 16 planes requested at a time
+  uint16_t* ts = smem;
+  const int TSR = a.Rpad + 8;  // padded row: 16-byte fragment reads of 32 rows spread over the banks
+  const int quads = a.Rpad >> 2;
+  for (int e = tid; e < MT * 32 * quads; e += 512) {
+    const int row = e / quads, c = (e - row * quads) * 4;
+    f32x4_t t = {0.f, 0.f, 0.f, 0.f};
+    if (ready && row < rows) {
+      constexpr int PB = MT == 1 ? 8 : 16;  // planes requested at a time
+      for (int p0 = 0; p0 < a.n_lora_slices; p0 += PB) {
+        u32x4_t v[PB];
+#pragma unroll
+        for (int u = 0; u < PB; ++u) {
+          const int p = p0 + u < a.n_lora_slices ? p0 + u : a.n_lora_slices - 1;
+          v[u] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rp, (int)((((size_t)p * a.M + row) * a.ldt + c) * 4), 0, 0x10));
+        }
+#pragma unroll
+        for (int u = 0; u < PB; ++u)
+          if (p0 + u < a.n_lora_slices) t += __builtin_bit_cast(f32x4_t, v[u]);
+      }
+    }
+    uint2 pk;
+    pk.x = pack_bf2(t[0], t[1]);
+    pk.y = pack_bf2(t[2], t[3]);
+    *reinterpret_cast<uint2*>(ts + row * TSR + c) = pk;
+  }
+  __syncthreads();
+  // delta^T = B^T . t^T: with the B columns as the MFMA A operand and the t rows as its B operand a lane ends
+  // up with 16 columns of ONE row, four adjacent ones per register group, which leave as 8-byte stores
+  const bool vec_t = (a.lora_r & 7) == 0;  // whole 8-rank groups: one 16-byte LDS read per fragment
+  for (int i = 0, tile = tile0; tile < ntiles; ++i, tile += tstride) {
+    const int n = tile * 32 + nl;
+    const int seg = tile * 32 >= a.seg_end[0] ? (tile * 32 >= a.seg_end[1] ? 2 : 1) : 0;  // host: ends are multiples of 32
+    const int toff = seg * a.lora_r;
+    bf16x8_t tbf = tb0[0];
+#pragma unroll
+    for (int q = 1; q < PT; ++q)
+      if (i == q) tbf = tb0[q];
+    // one row tile at a time (the stage must not raise the register count of the multiply loop)
+#pragma unroll 1
+    for (int m = 0; m < MT; ++m) {
+      if (m * 32 >= a.M) break;
+      f32x16_t dl;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dl[r] = 0.f;
+#pragma unroll 1
+      for (int ks = 0; ks < ksteps; ++ks) {
+        const int k0 = ks * 16 + h * 8;
+        bf16x8_t tb = tbf, ta;
+        if (vec_t) {
+          u32x4_t z = {0u, 0u, 0u, 0u};
+          if (k0 < a.lora_r) z = *reinterpret_cast<const u32x4_t*>(ts + (m * 32 + nl) * TSR + toff + k0);
+          ta = __builtin_bit_cast(bf16x8_t, z);
+        } else {
+          uint16_t tz[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) tz[j] = k0 + j < a.lora_r ? ts[(m * 32 + nl) * TSR + toff + k0 + j] : (uint16_t)0;
+          __builtin_memcpy(&ta, tz, 16);
+        }
+        if (ks > 0) {
+          uint16_t bz[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) bz[j] = k0 + j < a.lora_r ? a.lora_b[(size_t)(k0 + j) * a.N + n] : (uint16_t)0;
+          __builtin_memcpy(&tb, bz, 16);
+        }
+        dl = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tb, ta, dl, 0, 0, 0);
+      }
+      // register r of lane (row nl, h): column (r >> 2) * 8 + h * 4 + (r & 3) of the tile
+      const int row = m * 32 + nl;
+      if (row < a.M) {
+        uint16_t* dst = a.delta + (size_t)row * a.N + tile * 32 + h * 4;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 pk;
+          pk.x = pack_bf2(rbf(rbf(dl[4 * g]) * a.lora_ls), rbf(rbf(dl[4 * g + 1]) * a.lora_ls));
+          pk.y = pack_bf2(rbf(rbf(dl[4 * g + 2]) * a.lora_ls), rbf(rbf(dl[4 * g + 3]) * a.lora_ls));
+          *reinterpret_cast<uint2*>(dst + g * 8) = pk;
+        }
+      }
+    }
+  }
+  // the last block to finish puts the counters back
+  __syncthreads();
+  if (tid == 0) {
+    const uint32_t old = __hip_atomic_fetch_add(a.sync + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old == (uint32_t)(L - 1)) {
+      __hip_atomic_store(a.sync + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(a.sync + 0, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
 template <int MT, bool LORA>
 __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* smem) {
   constexpr int TS = KD::TS, TPW = KD::TPW, XS = KD::XS, ROWS = MT * 32;
@@ -1205,7 +1349,12 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
   const int kb0 = slice * per;
   const int kb1 = (kb0 + per < KT) ? kb0 + per : KT;
   const int nsteps = (kb1 - kb0) / TS, last_step = nsteps - 1;  // host: whole steps
-  if (nsteps <= 0) return;
+  if (nsteps <= 0) {
+    if constexpr (LORA) {
+      if (a.delta) lora_delta_stage<MT>(a, smem, false);
+    }
+    return;
+  }
   const int gs = __builtin_ctz(a.G >> 6), KG = a.K / a.G;
   const int NT = LORA ? (a.Rpad >> 5) : (a.N >> 5);
   const int nb = LORA ? ct : (int)blockIdx.x * 4 + ct;
@@ -1325,21 +1474,37 @@ __device__ __forceinline__ void gemm_block_dma(const QLinearArgs& a, uint16_t* s
       }
   }
   __syncthreads();
-  if (!tile_ok) return;
-  const int col = nb * 32 + nl;
+  const bool with_delta = LORA && a.delta != nullptr;
+  if (!tile_ok && !with_delta) return;
+  if (tile_ok) {
+    const int col = nb * 32 + nl;
+    const __amdgpu_buffer_rsrc_t rtp = make_rsrc(a.t_part, 0x7FFFFFFFu);
 #pragma unroll
-  for (int m = 0; m < MT; ++m)
+    for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int r8 = 0; r8 < 8; ++r8) {
-      const int r = kw ? r8 + 8 : r8;
-      const int row = m * 32 + acc_row(r, lane);
-      if (row >= a.M) continue;
-      const float mine = kw ? acc[m][r8 + 8] : acc[m][r8], other = hb[(((ct * MT + m) * 16 + r) << 6) + lane];
-      const float v = kw ? other + mine : mine + other;  // first half + second half
-      if (LORA) a.t_part[((size_t)slice * a.M + row) * a.ldt + col] = v;
-      else if (a.y_bf16) a.y_bf16[(size_t)row * a.ldy + col] = f2bf(v);
-      else a.y_part[((size_t)slice * a.M + row) * a.N + col] = v;
+      for (int r8 = 0; r8 < 8; ++r8) {
+        const int r = kw ? r8 + 8 : r8;
+        const int row = m * 32 + acc_row(r, lane);
+        if (row >= a.M) continue;
+        const float mine = kw ? acc[m][r8 + 8] : acc[m][r8], other = hb[(((ct * MT + m) * 16 + r) << 6) + lane];
+        const float v = kw ? other + mine : mine + other;  // first half + second half
+        if (LORA) {
+          const size_t idx = ((size_t)slice * a.M + row) * a.ldt + col;
+          if (with_delta) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rtp, (int)(idx * 4), 0, 0x10);
+          else a.t_part[idx] = v;
+        } else if (a.y_bf16) {
+          a.y_bf16[(size_t)row * a.ldy + col] = f2bf(v);
+        } else {
+          a.y_part[((size_t)slice * a.M + row) * a.N + col] = v;
+        }
+      }
+  }
+  if constexpr (LORA) {
+    if (with_delta) {
+      __syncthreads();  // every wave is done with the exchange area before t is staged there
+      lora_delta_stage<MT>(a, smem, true);
     }
+  }
 }
 
 template <int MT>
@@ -1765,9 +1930,37 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
 // Host-side dispatch shared by the C entry point and the decode-step launcher.
 // Output: y_bf16 [M, N] when nsplit == 1 and y_bf16 != null, else y_part
 // [nsplit][M][N] f32 planes.  t_part: [qlinear_num_lora_splits(K, N)][M][ldt] f32.
+size_t qlinear_delta_sync_bytes(int M, int Rpad) {
+  // hand-over state (3 words, 256 bytes reserved) | t bf16 [rows rounded up to 32][Rpad]
+  return 256 + (size_t)((M + 31) / 32 * 32) * Rpad * 2;
+}
+
+static bool dma_shape(int M, int K, int N, int Rpad, int nsplit, bool lora) {
+  const int KT = K / 64;
+  return M <= 128 && !four_wave(K, N) && K % 256 == 0 && slices_ok(KT, nsplit) && slice_len(KT, nsplit) % 4 == 0 &&
+         (!lora || lora_slice_len(K, N) % 4 == 0) && (size_t)K * N / 2 < (1u << 31) && (size_t)K * Rpad * 2 < (1u << 31);
+}
+
+bool qlinear_delta_ok(int M, int K, int N, int Rpad, int r, int nsplit) {
+  if (M <= 0 || K % 64 || N % 32 || nsplit < 1 || nsplit > TMX_MAX_SPLITS) return false;
+  if (r <= 0 || r > 64 || Rpad <= 0 || Rpad % 32 || Rpad > 128) return false;
+  if (!dma_shape(M, K, N, Rpad, nsplit, true)) return false;
+  // every workgroup of the launch is resident at once (the LoRA blocks wait for one another): one per CU
+  // at 128 rows, two below
+  const int nls = qlinear_num_lora_splits(K, N);
+  const int lbps = (nls + nsplit - 1) / nsplit;
+  const int blocks = ((N + 127) / 128 + lbps) * nsplit;
+  if (blocks > (M > 64 ? 256 : 512) || (size_t)M * N * 2 >= (1u << 31)) return false;
+  // The stage is a chain of round trips behind the LoRA blocks' own slices (arrive, wait, sum of the planes,
+  // tiles: 6 to 10 us); it stays hidden only behind main blocks of at least 8 steps, and with at most two
+  // column tiles per wave.  Shorter projections (measured: q|k|v and o of the 8B shape, 4 steps, 14.5 -> 21 us and
+  // 13 -> 15.4 us per launch) keep the LoRA product in their consumer.
+  return slice_len(K / 64, nsplit) >= 32 && N / 32 <= lbps * nsplit * 8 * 2;
+}
+
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
-                 int N, int G, int Rpad, int nsplit) {
+                 int N, int G, int Rpad, int nsplit, const LoraDelta* ld) {
   if (!x || !qw || !scales || (!y_bf16 && !y_part)) return TMX_ERR_ARG;
   if (M <= 0 || K <= 0 || N <= 0) return TMX_ERR_SHAPE;
   if (K % 64 || N % 32 || G % 64 || (G & (G - 1)) || K % G || (ldx % 8)) return TMX_ERR_SHAPE;
@@ -1793,6 +1986,20 @@ int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const v
   const int nls = qlinear_num_lora_splits(K, N);
   a.lora_blocks_per_split = (nls + nsplit - 1) / nsplit;
   a.kt_per_lora_split = lora_slice_len(K, N);
+  if (ld) {
+    // the LoRA blocks also produce delta = bf16(bf16(t . B) * ls): only the direct-to-LDS kernel does that
+    if (!a_t || !ld->delta || !ld->lora_b || !ld->sync_ws) return TMX_ERR_ARG;
+    if (!qlinear_delta_ok(M, K, N, Rpad, ld->r, nsplit) || (size_t)M * ldx * 2 >= (1u << 31)) return TMX_ERR_UNSUPPORTED;
+    for (int i = 0; i < 3; ++i)
+      if (ld->seg_end[i] % 32) return TMX_ERR_SHAPE;
+    a.delta = ld->delta;
+    a.lora_b = ld->lora_b; a.lora_r = ld->r; a.lora_ls = ld->ls;
+    a.seg_end[0] = ld->seg_end[0]; a.seg_end[1] = ld->seg_end[1]; a.seg_end[2] = ld->seg_end[2];
+    a.sync = (uint32_t*)ld->sync_ws;
+    a.sync_t16 = (uint16_t*)((char*)ld->sync_ws + 256);
+    a.sync_status = ld->status;
+    a.n_lora_slices = (KT + a.kt_per_lora_split - 1) / a.kt_per_lora_split;  // slices that hold k-tiles
+  }
   if (M > 128) {
     // more than 128 rows: the 256-row block (whole 2-tile steps, 32-bit byte offsets per row block)
     if (K % 128 || a.kt_per_split % 2 || (a_t && a.kt_per_lora_split % 2) || (size_t)256 * ldx * 2 >= (1u << 31) ||
@@ -1942,6 +2149,26 @@ extern "C" int tmx_qlora_linear_planes(void* stream, const void* x, const void* 
                                        float* t_part, int M, int K, int N, int G, int r_pad, int nsplit) {
   return qlinear_base((hipStream_t)stream, x, K, qweight, scales, lora_a_t, nullptr, y_part, t_part,
                       TMX_MAX_RPAD, M, K, N, G, r_pad, nsplit);
+}
+
+extern "C" size_t tmx_qlora_linear_delta_workspace_bytes(int M, int K, int N, int r, int r_pad, int nsplit) {
+  return qlinear_delta_ok(M, K, N, r_pad, r, nsplit) ? qlinear_delta_sync_bytes(M, r_pad) : 0;
+}
+
+extern "C" int tmx_qlora_linear_planes_delta(void* stream, const void* x, const void* qweight, const void* scales,
+                                             const void* lora_a_t, const void* lora_b, float* y_part, float* t_part,
+                                             void* delta, void* workspace, int M, int K, int N, int G, int r,
+                                             int r_pad, float lora_scale, int seg_end0, int seg_end1, int nsplit) {
+  if (!lora_a_t || !lora_b || !delta || !workspace) return TMX_ERR_ARG;
+  LoraDelta ld = {};
+  ld.delta = (uint16_t*)delta;
+  ld.lora_b = (const uint16_t*)lora_b; ld.r = r; ld.ls = lora_scale;
+  ld.seg_end[0] = seg_end0; ld.seg_end[1] = seg_end1; ld.seg_end[2] = N;
+  ld.sync_ws = workspace;
+  int rc = zero_words((hipStream_t)stream, (uint32_t*)workspace, 64);
+  if (rc != TMX_OK) return rc;
+  return qlinear_base((hipStream_t)stream, x, K, qweight, scales, lora_a_t, nullptr, y_part, t_part, TMX_MAX_RPAD, M, K, N, G,
+                      r_pad, nsplit, &ld);
 }
 
 extern "C" int tmx_qlora_linear(void* stream, const void* x, const void* qweight, const void* scales,

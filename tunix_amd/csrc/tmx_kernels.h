@@ -39,7 +39,27 @@ struct QLinearArgs {
   float* sync_part;
   uint16_t* sync_t16;
   int sync_blocks;
+  // LoRA delta by the LoRA blocks of a split projection (direct-to-LDS kernel): once every slice of
+  // x . A has arrived (sync, sync_t16 as above; lora_b, lora_r, lora_ls, seg_end as above), the LoRA
+  // blocks share the columns of delta = bf16(bf16(t . B) * ls), [M][N] bf16, which the consumer adds
+  // to the rounded sum of the planes instead of multiplying by B itself
+  uint16_t* delta;
+  int n_lora_slices;       // slices that hold k-tiles (the launch may have a few more LoRA blocks)
 };
+
+// What qlinear_base needs to let the LoRA blocks produce the delta (all or nothing).
+struct LoraDelta {
+  uint16_t* delta;         // [M][N] bf16 out
+  const uint16_t* lora_b;  // [r][N]
+  int r;
+  float ls;
+  int seg_end[3];          // column ends of the fused matrices (multiples of 32)
+  void* sync_ws;           // qlinear_delta_sync_bytes(M, Rpad) bytes, first 16 zero between launches (the kernel leaves them so)
+  uint32_t* status;        // may be null
+};
+size_t qlinear_delta_sync_bytes(int M, int Rpad);
+// true when qlinear_base(..., &ld) with these shapes runs the kernel that fills ld.delta
+bool qlinear_delta_ok(int M, int K, int N, int Rpad, int r, int nsplit);
 
 // Routed experts (Qwen3 MoE): one launch multiplies, for every expert, the rows routed to it.
 struct MoeArgs {
@@ -88,6 +108,7 @@ struct RowNormArgs {
   const float* y_part;          // [nsplit][M][D] f32 planes
   int nsplit;
   LoraIn lora;
+  const uint16_t* delta;        // [M, D] bf16 LoRA delta made by the projection (replaces lora), or null
   const uint16_t* moe_y;        // [M * top_k, D] routed-expert outputs (replaces y when set)
   const float* moe_w;           // [M * top_k] routing weights
   int top_k;
@@ -279,6 +300,6 @@ int qlinear_wide_lora(hipStream_t st, const void* x, int ldx, const void* qw, co
                       uint16_t* t16, int M, int K, int N, int G, int Rpad);
 int qlinear_base(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                  const void* a_t, void* y_bf16, float* y_part, float* t_part, int ldt, int M, int K,
-                 int N, int G, int Rpad, int nsplit);
+                 int N, int G, int Rpad, int nsplit, const LoraDelta* ld = nullptr);
 
 }  // namespace tmx
