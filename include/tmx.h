@@ -9,7 +9,12 @@
  * Conventions
  *   - every pointer is a DEVICE pointer unless its name ends in _host;
  *   - `stream` is a hipStream_t passed as void*; entry points only enqueue work
- *     on it: they never allocate, free or synchronise;
+ *     on it: they never allocate, free or synchronise.  Three calls at the end of
+ *     this file wait for the stream and say so where they are declared:
+ *     tmx_decode_status, tmx_decode_steps_graph (which also creates and destroys
+ *     a stream, an event and a graph) and tmx_decode_steps_profiled (events);
+ *     some kernels set their dynamic LDS limit with hipFuncSetAttribute on their
+ *     first launch in the process;
  *   - bf16 tensors are raw 16-bit patterns, row-major, innermost index last;
  *   - return value: TMX_OK or a negative TMX_ERR_* code, nothing is launched
  *     when an argument check fails.
