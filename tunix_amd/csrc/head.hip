@@ -339,7 +339,7 @@ __global__ __launch_bounds__(512, 1) void head_wide_kernel(HeadArgs a, int tok_b
     step = step < last_step ? step : last_step;
     uint16_t* base = smem + (size_t)buf * ROWS * XS + wave * 4 * XS;
 #pragma unroll
-    for (int i = 0; i < XR; ++i) load_row_to_lds(rw, base + i * 32 * XS, woff[i], step * (TS * 128));
+    for (int i = 0; i < XR; ++i) load_row_to_lds_nt(rw, base + i * 32 * XS, woff[i], step * (TS * 128));
   };
   constexpr int kYounger = 4 * TS;
   auto wait_slab = [&]() __attribute__((always_inline)) {

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kSbThreads) void sb_linear_kernel(SbLinearArgs a) {
   for (int i = 0; i < kSbMaxTiles; ++i) {
     if (i < per) {
       const int kt = min(kt0 + i, KT - 1);
-      wr[i] = wsrc[(size_t)kt * 64];
+      wr[i] = __builtin_nontemporal_load(wsrc + (size_t)kt * 64);  // every tile is read once, by this wave
       sr[i] = ssrc[(size_t)(kt >> gs) * 32];
     }
   }
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(kSbThreads) void sb_linear_kernel(SbLinearArgs a) {
         const uint32_t wd[4] = {wr[i].x, wr[i].y, wr[i].z, wr[i].w};
         if (base + i + kSbMaxTiles < per) {  // slot consumed: refill it for the tile 8 further on
           const int ktn = min(kt + kSbMaxTiles, KT - 1);
-          wr[i] = wsrc[(size_t)ktn * 64];
+          wr[i] = __builtin_nontemporal_load(wsrc + (size_t)ktn * 64);
           sr[i] = ssrc[(size_t)(ktn >> gs) * 32];
         }
 #pragma unroll

@@ -147,6 +147,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 __device__ __forceinline__ void load_row_to_lds(__amdgpu_buffer_rsrc_t r, void* dst, int voffset, int soffset) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16, voffset, soffset, 0, 0);
 }
+// the same with the non-temporal cache policy, for data that is read once
+__device__ __forceinline__ void load_row_to_lds_nt(__amdgpu_buffer_rsrc_t r, void* dst, int voffset, int soffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16, voffset, soffset, 0, 2);
+}
 
 
 inline int check_launch() {
