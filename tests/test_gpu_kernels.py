@@ -684,7 +684,7 @@ def test_moe_experts_match_oracle(B, D, F, E, k, group):
 ])
 def test_projection_writes_the_lora_delta(M, K, widths, group, r, nsplit):
   """tmx_qlora_linear_planes_delta: the y planes add up to x . W as before, and delta equals
-  bf16(bf16(t . B) * s) with t = bf16(x . A) per fused matrix (tunix's qwix-wrapped Einsum, SURVEY a16:
+  bf16(bf16(t . B) * s) with t = bf16(x . A) per fused matrix (tunix's qwix-wrapped Einsum, tunix/models/llama3/model.py:216-218:
   (x . A) . B * alpha / rank), twice in a row on one workspace (its counters must be back at zero)."""
   T = G.Keep()
   lib = _lib.lib()
