@@ -34,6 +34,8 @@ WORKLOADS = {
     'qwen3-30b-a3b-moe': ('qwen3_30b_a3b', 32, 256, 512, 64, 8, 0.9, 1.0),
 }
 ATTN_ONLY_LORA = {'qwen3-30b-a3b-moe'}
+LABELS = {'llama3.1-8b-grpo': '8B', 'llama3.2-1b-b1': '1B single-sequence', 'toy': 'toy',
+          'qwen3-8b-b128': 'Qwen3-8B 128-sequence', 'qwen3-30b-a3b-moe': 'Qwen3-30B-A3B MoE'}
 
 CLASS_NAMES = ['row_norm', 'qkv_linear', 'rope_kvwrite', 'attention', 'o_linear', 'gate_up_linear',
                'swiglu', 'down_linear', 'head_sample', 'advance_step', 'empty_launch', 'router']
@@ -159,7 +161,6 @@ def main():
   from tunix_amd.configs import CacheConfig
   from tunix_amd.model import ModelConfig, QLoRAModel
   from tunix_amd.sampler import Sampler
-  sys.path.insert(0, os.path.join(ROOT, 'tests'))
 
   name, batch, prompt, new, group, rank, temp, top_p = WORKLOADS[args.workload]
   if args.sequences > 0:
@@ -262,9 +263,11 @@ def main():
   assert bool(((toks >= 0) & (toks < cfg.vocab_size)).all().item())
   lps = st['logprobs'][:, start:start + args.warmup + args.steps]
   assert bool(torch.isfinite(lps).all().item()) and bool((lps <= 0).all().item())
+  # a hand-over inside a launch whose bounded wait ran out would have dropped a LoRA term: raises if so
+  sampler.check_device_status(st)
 
   result = {
-      'metric': 'generated tokens/s at 1 GPU, int4 QLoRA 8B rollout (decode)',
+      'metric': f'generated tokens/s at 1 GPU, int4 QLoRA {LABELS[args.workload]} rollout (decode)',
       'value': batch * args.steps / dt,
       'unit': 'tokens/s',
       'n_gpus': 1,
@@ -323,6 +326,8 @@ def main():
       tot_ms += ms
       tot_cnt += cnt
       done_steps += 1
+    sampler.check_device_status(st)  # the profiled steps too
+    result['device_status'] = 'ok: no bounded in-kernel wait ran out (timed window and profiled replay)'
     per_step = tot_ms / max(ctx_n, 1)
     result['kernel_ms_per_step'] = {n: round(float(v), 4) for n, v in zip(CLASS_NAMES, per_step)}
     layer0 = model.layers[0]
@@ -336,6 +341,17 @@ def main():
     }
     if not cfg.num_experts and tot_cnt[CLASS_NAMES.index('swiglu')] == 0:
       alg['gate_up_linear'] -= batch * cfg.hidden_dim * 2  # fused SwiGLU: [M, F] goes out, not [M, 2 F]
+    # multiply-add work of the dense projections (2 M K N, + the LoRA products): above the ridge of
+    # 2.5 PFLOP/s / 8 TB/s = 312 flop per byte a kernel is priced against the bf16 MFMA peak instead
+    def linear_flops(pl):
+      f = 2.0 * batch * pl.k * pl.n
+      if pl.lora_a_t is not None:
+        f += 2.0 * batch * pl.rank * (pl.k * len(pl.seg_cols) + pl.n)
+      return f
+    flops = {}
+    if not cfg.num_experts:
+      flops = {'qkv_linear': linear_flops(layer0['qkv']), 'o_linear': linear_flops(layer0['o']),
+               'gate_up_linear': linear_flops(layer0['gate_up']), 'down_linear': linear_flops(layer0['down'])}
     # kernel symbols (as rocprofv3 names them) and the launch classes each one serves
     mt = 1 if batch <= 32 else (2 if batch <= 64 else 4)
     # K % 256 == 0 below 8192 with fewer than 16 column blocks runs the 4-wave kernel, the rest the
@@ -355,7 +371,8 @@ def main():
         if batch <= 64 and gu.k % 512 == 0:   # 8 waves per workgroup, activation slab by direct-to-LDS loads
           # LoRA mode: 0 none, 1 every workgroup multiplies x by A itself, 2 a few workgroups do it once and
           # hand t over (K / 256 <= 32 producers that fit beside the F / 64 main workgroups within 256)
-          mode = 0 if not lora else (2 if gu.k // 256 <= 32 and cfg.hidden_dim // 64 + gu.k // 256 <= 256 else 1)
+          cus = torch.cuda.get_device_properties(0).multi_processor_count
+          mode = 0 if not lora else (2 if gu.k // 256 <= 32 and cfg.hidden_dim // 64 + gu.k // 256 <= cus else 1)
           sym = f'tmx::qlinear_gate_up8_kernel<{mt}, {mode}>'
         else:
           sym = f'tmx::qlinear_gate_up_kernel<{mt}>' if lora else f'tmx::qlinear_mfma4_kernel<{mt}>'
@@ -405,17 +422,25 @@ def main():
       byts = float(sum(alg[c] * launches_per_class[c] for c in classes)) / n
       avg = t / n
       per_symbol[sym] = {'classes': classes, 'total_ms_per_step': avg * n / max(ctx_n, 1), 'launches_per_step': n / max(ctx_n, 1),
-                         'avg_launch_ms': avg,
+                         'avg_launch_ms': avg, 'bound': 'hbm',
                          'algorithmic_bytes_per_launch': byts,
                          'achieved_GBps': byts / (avg * 1e-3) / 1e9, 'frac': byts / (avg * 1e-3) / 8e12}
+      if all(c in flops for c in classes):
+        fl = float(sum(flops[c] * launches_per_class[c] for c in classes)) / n
+        per_symbol[sym].update({'flops_per_launch': fl, 'achieved_TFLOPs': fl / (avg * 1e-3) / 1e12,
+                                'frac_of_2500_TFLOPs': fl / (avg * 1e-3) / 2.5e15})
+        if fl / byts > 2.5e15 / 8e12:
+          per_symbol[sym]['bound'] = 'mfma'
     dom = max(per_symbol, key=lambda k: per_symbol[k]['total_ms_per_step'])
     traffic = None
     tpath = os.path.join(ROOT, 'profiles', 'traffic.json')
     if os.path.exists(tpath):  # HBM bytes per launch from the rocprofv3 --pmc runs (see profiles/)
       traffic = json.load(open(tpath)).get(args.workload, {}).get(dom)
     d = per_symbol[dom]
-    result['roofline'] = {'bound': 'hbm', 'achieved': d['achieved_GBps'], 'peak': 8000.0, 'unit': 'GB/s',
-                          'frac': d['frac'], 'traffic': traffic, 'kernel': dom,
+    mf = d['bound'] == 'mfma'
+    result['roofline'] = {'bound': d['bound'], 'achieved': d['achieved_TFLOPs'] if mf else d['achieved_GBps'],
+                          'peak': 2500.0 if mf else 8000.0, 'unit': 'TFLOP/s' if mf else 'GB/s',
+                          'frac': d['frac_of_2500_TFLOPs'] if mf else d['frac'], 'traffic': traffic, 'kernel': dom,
                           'avg_launch_ms': d['avg_launch_ms'],
                           'empty_launch_event_pair_ms': pair_ms,
                           'algorithmic_bytes_per_launch': d['algorithmic_bytes_per_launch'],

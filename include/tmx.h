@@ -9,8 +9,8 @@
  * Conventions
  *   - every pointer is a DEVICE pointer unless its name ends in _host;
  *   - `stream` is a hipStream_t passed as void*; entry points only enqueue work
- *     on it: they never allocate, free or synchronise.  Three calls at the end of
- *     this file wait for the stream and say so where they are declared:
+ *     on it: they never allocate, free or synchronise.  Four calls wait for the
+ *     stream and say so where they are declared: tmx_handover_status,
  *     tmx_decode_status, tmx_decode_steps_graph (which also creates and destroys
  *     a stream, an event and a graph) and tmx_decode_steps_profiled (events);
  *     some kernels set their dynamic LDS limit with hipFuncSetAttribute on their
@@ -121,12 +121,20 @@ int tmx_qlora_linear_planes(void* stream, const void* x, const void* qweight, co
  * projections whose K-slices are long enough to hide it (slices of at least 2048 rows of W, at most two
  * 32-column tiles per LoRA wave): tmx_qlora_linear_delta_workspace_bytes returns 0 for every other shape
  * and the call TMX_ERR_UNSUPPORTED.  workspace: that many bytes (cleared by the call: one small launch).
- * Up to 128 rows, r <= 64.  No counterpart in the reference beyond the LoRA arithmetic itself. */
+ * Up to 128 rows, r <= 64.  The LoRA workgroups wait for one another a bounded number of polls; if that
+ * wait ever runs out they take t as zero and set a word inside `workspace` that tmx_handover_status
+ * reports.  No counterpart in the reference beyond the LoRA arithmetic itself. */
 size_t tmx_qlora_linear_delta_workspace_bytes(int M, int K, int N, int r, int r_pad, int nsplit);
 int tmx_qlora_linear_planes_delta(void* stream, const void* x, const void* qweight, const void* scales,
                                   const void* lora_a_t, const void* lora_b, float* y_part, float* t_part,
                                   void* delta, void* workspace, int M, int K, int N, int G, int r, int r_pad,
                                   float lora_scale, int seg_end0, int seg_end1, int nsplit);
+
+/* WAITS for `stream`, then reports and clears the "a bounded wait ran out" word of a hand-over workspace
+ * (the `workspace` of tmx_qlora_linear_planes_delta or tmx_qlora_gate_up_swiglu_handover): TMX_OK, or
+ * TMX_ERR_DEVICE_WAIT when the last call on that workspace dropped its LoRA term.  No counterpart in
+ * the reference (XLA has no such failure mode). */
+int tmx_handover_status(void* stream, void* workspace);
 
 /* One projection of the single-sequence regime (1..4 rows) in ONE launch: optional RMSNorm of
  * x in the prologue (norm_w != NULL; family as tmx_rmsnorm), the int4 product, the LoRA delta
@@ -188,6 +196,18 @@ int tmx_swiglu(void* stream, const void* gate_up_bf16, const float* gate_up_part
 int tmx_qlora_gate_up_swiglu(void* stream, const void* x, const void* qweight, const void* scales,
                              const void* lora_a_t, const void* lora_b, void* act, int M, int K, int F,
                              int G, int r, float lora_scale);
+
+/* The same launch in the form the decode step runs at up to 64 rows with LoRA: t = x . [A_gate | A_up] is
+ * computed once, by K / 256 extra workgroups of the launch, and handed to the others through `workspace`
+ * (tmx_qlora_gate_up_swiglu_handover_bytes(M, K, F, r) bytes, whose state block the call clears with one
+ * small launch) instead of being recomputed by every workgroup; same results up to the summation order of
+ * t's K-slices.  The size query returns 0, and the call TMX_ERR_UNSUPPORTED, for shapes that do not take
+ * this form on the current device (more than 64 rows, K % 512 != 0, 2 r > 32, or more workgroups than
+ * compute units).  The receiving workgroups wait a bounded number of polls: see tmx_handover_status. */
+size_t tmx_qlora_gate_up_swiglu_handover_bytes(int M, int K, int F, int r);
+int tmx_qlora_gate_up_swiglu_handover(void* stream, const void* x, const void* qweight, const void* scales,
+                                      const void* lora_a_t, const void* lora_b, void* act, void* workspace,
+                                      int M, int K, int F, int G, int r, float lora_scale);
 
 /* ---- GQA decode attention -------------------------------------------------- */
 

@@ -61,8 +61,9 @@ def test_projection_of_one_hot_rows_is_a_row_lookup(K, N, group):
                       min_exact=0.99, what=f'one-hot {K}x{N}')
 
 
-@pytest.mark.parametrize('M,r', [(64, 16), (64, 0), (17, 16)])
-def test_fused_gate_up_of_one_hot_rows_is_swiglu_of_a_row_lookup(M, r):
+@pytest.mark.parametrize('M,r,handover', [(64, 16, False), (64, 0, False), (17, 16, False),
+                                          (64, 16, True), (33, 16, True), (17, 16, True)])
+def test_fused_gate_up_of_one_hot_rows_is_swiglu_of_a_row_lookup(M, r, handover):
   """gate | up + LoRA + SwiGLU in one launch at the 8B shape (K = 4096, F = 14336): with one-hot
   activation rows the two projections are rows of the bit-exactly dequantised matrix, so the
   activation is known in closed form."""
@@ -81,8 +82,17 @@ def test_fused_gate_up_of_one_hot_rows_is_swiglu_of_a_row_lookup(M, r):
   x = torch.zeros(M, K, dtype=torch.bfloat16, device=G.DEV)
   x[torch.arange(M), ks] = amp.to(torch.bfloat16)
   act = torch.empty(M, F, dtype=torch.bfloat16, device=G.DEV)
-  G.call('tmx_qlora_gate_up_swiglu', S(), G.p(x), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t), G.p(pl.lora_b),
-         G.p(act), M, K, F, group, r, 2.0)
+  if handover:
+    # the form the decode step runs: x . A once per launch by 16 (8 up to 32 rows) extra workgroups
+    nb = _lib.lib().tmx_qlora_gate_up_swiglu_handover_bytes(M, K, F, r)
+    assert nb > 0
+    wsb = torch.empty(nb, dtype=torch.uint8, device=G.DEV)
+    G.call('tmx_qlora_gate_up_swiglu_handover', S(), G.p(x), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t),
+           G.p(pl.lora_b), G.p(act), G.p(wsb), M, K, F, group, r, 2.0)
+    G.call('tmx_handover_status', S(), G.p(wsb))
+  else:
+    G.call('tmx_qlora_gate_up_swiglu', S(), G.p(x), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t), G.p(pl.lora_b),
+           G.p(act), M, K, F, group, r, 2.0)
   G.sync()
   y = _bf16_round(dense[ks].float() * amp[:, None])            # [M, 2F], exact
   slack = torch.zeros_like(y)                                  # how far a last-bit flip of the LoRA sum can move y

@@ -273,9 +273,79 @@ def test_fused_gate_up_swiglu_matches_oracle(M, K, F, group, r):
               M, K, F + 32, group, 0, 0.0) != 0
 
 
+@pytest.mark.parametrize('M,K,F,group,r', [
+    (5, 1024, 256, 64, 8), (32, 512, 128, 64, 16), (33, 2048, 512, 64, 16), (48, 4096, 256, 128, 16),
+    (64, 1024, 1024, 64, 16), (64, 4096, 1024, 64, 12),
+])
+def test_fused_gate_up_handover_matches_oracle(M, K, F, group, r):
+  """tmx_qlora_gate_up_swiglu_handover: the form of the fused gate | up launch that the decode step runs with
+  LoRA at up to 64 rows (x . A computed once by K / 256 extra workgroups and handed over through memory;
+  8 producers of 8 k-tiles up to 32 rows, 16 of 4 above) against the oracle's separate projections
+  (tunix/models/llama3/model.py:489-496), twice in a row on one workspace: its state must be back at zero."""
+  lib = _lib.lib()
+  rng = np.random.default_rng(M + K + F + 1)
+  x = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+  ws = [bf16_round(rng.standard_normal((K, F)).astype(np.float32) * 0.03) for _ in range(2)]
+  loras = [(bf16_round(rng.standard_normal((K, r)).astype(np.float32) * 0.03),
+            bf16_round(rng.standard_normal((r, F)).astype(np.float32) * 0.03)) for _ in range(2)]
+  pl = quant.PackedLinear.from_dense([torch.from_numpy(w) for w in ws], group, G.DEV,
+                                     [tuple(torch.from_numpy(m) for m in l) for l in loras], 2.0)
+  ys, flips = [], []
+  for i, w in enumerate(ws):
+    qo, so = int4.quantize(w, group)
+    lin = L.Linear(q=qo, scale=so, group=group, a=loras[i][0], b=loras[i][1], lora_scale=2.0)
+    ys.append(lin(x, BF16))
+    base = bf16_round(x @ lin.weight())
+    f = G.ulp_bf16(base) + 2.0 * G.ulp_bf16(ys[i] - base) + G.ulp_bf16(ys[i])
+    flips.append(f + 2.0 * (G.ulp_bf16(bf16_round(x @ loras[i][0])) @ np.abs(loras[i][1])))
+  ref = bf16_round(L.silu(ys[0], BF16) * ys[1])
+  nb = lib.tmx_qlora_gate_up_swiglu_handover_bytes(M, K, F, r)
+  assert nb > 0
+  wsb = torch.full((nb,), 0xAB, dtype=torch.uint8, device=G.DEV)  # the call clears the state block itself
+  xt = G.bf(x)
+  outs = []
+  for _ in range(2):
+    act = torch.full((M, F), float('nan'), dtype=torch.bfloat16, device=G.DEV)
+    G.call('tmx_qlora_gate_up_swiglu_handover', S(), G.p(xt), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t),
+           G.p(pl.lora_b), G.p(act), G.p(wsb), M, K, F, group, r, 2.0)
+    G.call('tmx_handover_status', S(), G.p(wsb))
+    outs.append(G.host(act))
+  np.testing.assert_array_equal(outs[0], outs[1])
+  assert int(wsb[:256].view(torch.int32).abs().sum().item()) == 0
+  extra = 2.5 * np.maximum(G.ulp_bf16(ref), G.ulp_bf16(ys[0]) * np.abs(ys[1]))
+  extra = np.maximum(extra, 1.1 * flips[0] * np.abs(ys[1]) + flips[1] * np.abs(L.silu(ys[0], BF16)) + G.ulp_bf16(ref))
+  G.assert_bf16_close(outs[1], ref, ulps=1.0, extra=extra, min_exact=0.97, what=f'gate_up hand-over {M}x{K}x{F}')
+  # and against the form in which every workgroup multiplies by A itself: the same t up to the order its K-slices are added in
+  act1 = torch.empty(M, F, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_qlora_gate_up_swiglu', S(), G.p(xt), G.p(pl.qweight), G.p(pl.scales), G.p(pl.lora_a_t),
+         G.p(pl.lora_b), G.p(act1), M, K, F, group, r, 2.0)
+  G.sync()
+  assert (G.host(act1) == outs[1]).mean() > 0.97
+
+
+def test_handover_status_word_and_shape_limits():
+  """tmx_handover_status reports a set "wait ran out" word once and clears it (the word is written here from
+  the host: no kernel is made to wait); shapes outside the hand-over form are refused with a zero size."""
+  lib = _lib.lib()
+  assert lib.tmx_qlora_gate_up_swiglu_handover_bytes(64, 4096, 14336, 16) > 0
+  assert lib.tmx_qlora_gate_up_swiglu_handover_bytes(65, 4096, 14336, 16) == 0   # more than 64 rows
+  assert lib.tmx_qlora_gate_up_swiglu_handover_bytes(64, 4096 + 256, 14336, 16) == 0  # K % 512
+  assert lib.tmx_qlora_gate_up_swiglu_handover_bytes(64, 4096, 14336, 17) == 0   # 2 r > 32
+  assert lib.tmx_qlora_gate_up_swiglu_handover_bytes(64, 4096, 64 * 300, 16) == 0  # more workgroups than compute units
+  assert lib.tmx_qlora_gate_up_swiglu_handover(S(), 1, 1, 1, 1, 1, 1, 1, 65, 4096, 14336, 64, 16, 2.0) == -4
+  ws = torch.zeros(1024, dtype=torch.uint8, device=G.DEV)
+  assert lib.tmx_handover_status(S(), G.p(ws)) == 0
+  ws[252:256] = torch.tensor([1, 0, 0, 0], dtype=torch.uint8, device=G.DEV)
+  assert lib.tmx_handover_status(S(), G.p(ws)) == -6
+  assert lib.tmx_handover_status(S(), G.p(ws)) == 0
+  assert lib.tmx_handover_status(S(), None) == -1
+
+
 @pytest.mark.parametrize('B,N,Kh,H,C,step', [
     (2, 4, 4, 64, 64, 40), (3, 8, 2, 64, 96, 95), (2, 8, 4, 64, 33, 0), (4, 32, 8, 128, 300, 257),
     (2, 8, 1, 128, 128, 100), (1, 32, 8, 64, 768, 700), (2, 16, 8, 128, 520, 519), (1, 4, 4, 128, 16, 7),
+    # the 8B Qwen3 workload's cache (512-token prompts + 1024 new tokens) near its end and at an early step
+    (3, 32, 8, 128, 1536, 1500), (2, 32, 8, 128, 1536, 513),
 ])
 def test_gqa_decode_attention(B, N, Kh, H, C, step):
   T = G.Keep()
@@ -597,7 +667,7 @@ def test_head_sampling_distribution_chi2():
 
 # ---- routed experts (Qwen3 MoE) ---------------------------------------------------------------
 
-@pytest.mark.parametrize('B,D,E,k', [(8, 256, 16, 4), (32, 512, 128, 8), (3, 256, 8, 1)])
+@pytest.mark.parametrize('B,D,E,k', [(8, 256, 16, 4), (32, 512, 128, 8), (3, 256, 8, 1), (32, 2048, 128, 8)])
 def test_moe_route_matches_oracle(B, D, E, k):
   T = G.Keep()
   rng = np.random.default_rng(B + E)
@@ -714,6 +784,7 @@ def test_projection_writes_the_lora_delta(M, K, widths, group, r, nsplit):
     outs.append(G.host(d))
   np.testing.assert_array_equal(outs[0], outs[1])
   assert int(wsb[:16].view(torch.int32).abs().sum().item()) == 0
+  assert lib.tmx_handover_status(S(), G.p(wsb)) == 0   # no LoRA block's wait ran out
   got = outs[1]
   want = np.concatenate([bf16_round(bf16_round(bf16_round(x @ a) @ b) * ls) for a, b in zip(As, Bs)], axis=1)
   # a last-bit flip of a t element (f32 summation order of x . A) moves the product by ulp(t) |B|

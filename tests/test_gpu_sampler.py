@@ -85,6 +85,53 @@ def test_wide_layer_with_the_projection_side_lora_delta_matches_oracle():
   _compare_greedy(out, ref, 6, 12, lp_extra=2.0 ** -5)
 
 
+_WIDE = {}
+
+
+def _wide_pair():
+  """One 8B-width layer with LoRA r16 on all seven projections, built once for the tests that share it."""
+  if not _WIDE:
+    cfg = OM.Config('llama3', 1, 512, 4096, 14336, 32, 128, 8, norm_eps=1e-5)
+    oracle, model = _pair(cfg, seed=22, rank=16, alpha=32.0,
+                          targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
+    _WIDE.update(cfg=cfg, oracle=oracle, sampler=_sampler(model, cfg, 16))
+  return _WIDE['cfg'], _WIDE['oracle'], _WIDE['sampler']
+
+
+@pytest.mark.parametrize('n_seq', [33, 48, 64])
+def test_wide_layer_at_33_to_64_sequences_matches_oracle(n_seq):
+  """The 8B-width layer at 33, 48 and 64 sequences: the row counts at which the decode step runs the
+  two-row-tile instantiations of its projection kernels, and the fused gate | up launch takes its LoRA
+  projection from 16 producer workgroups (tunix/models/llama3/model.py:367-410, :489-496).  Ragged,
+  left-padded prompts; greedy tokens and log-probs against the oracle."""
+  cfg, oracle, s = _wide_pair()
+  rng = np.random.default_rng(6 + n_seq)
+  prompts = [rng.integers(3, cfg.vocab_size, 2 + i % 3) for i in range(n_seq)]
+  ref = OSAM.generate(oracle, cfg, prompts, 3, 16, eos_ids=(-1,))
+  out = s(prompt_token_ids=prompts, max_generation_steps=3, return_logprobs=True, eos_tokens=[-1])
+  _compare_greedy(out, ref, n_seq, 2 * n_seq, lp_extra=2.0 ** -5)
+  if n_seq == 64:
+    _WIDE.clear()  # frees the device copy of the layer
+
+
+@pytest.mark.parametrize('n_seq,heads,kv_heads', [(1, 8, 2), (3, 8, 2), (1, 32, 8)])
+def test_small_batch_attention_over_several_context_splits_matches_oracle(n_seq, heads, kv_heads):
+  """One to three sequences with ~600-token left-padded prompts in a 768-slot cache: the small-batch step
+  walks the context in 6 splits per kv head and merges them in the o projection's prologue
+  (tunix/models/llama3/model.py:367-410 with the mask of tunix/generate/utils.py:35-59).  8 greedy steps
+  against the oracle, log-probs included."""
+  cfg = OM.Config('llama3', 2, 512, 256, 512, heads, 64, kv_heads, norm_eps=1e-5)
+  oracle, model = _pair(cfg, seed=23 + n_seq, rank=16, alpha=32.0,
+                        targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
+  rng = np.random.default_rng(7 + n_seq)
+  prompts = [rng.integers(3, 512, n) for n in (600, 437, 590)[:n_seq]]
+  ref = OSAM.generate(oracle, cfg, prompts, 8, 768, eos_ids=(-1,))
+  out = _sampler(model, cfg, 768)(prompt_token_ids=prompts, max_generation_steps=8, return_logprobs=True,
+                                  eos_tokens=[-1])
+  np.testing.assert_array_equal(out.padded_prompt_tokens, ref['padded_prompt_tokens'])
+  _compare_greedy(out, ref, n_seq, 5 * n_seq)
+
+
 def test_left_padded_ragged_prompts_and_all_lora_targets():
   cfg = OM.Config('llama3', 2, 512, 256, 512, 8, 64, 2, norm_eps=1e-5)  # GQA group of 4
   oracle, model = _pair(cfg, seed=3, rank=16, alpha=32.0,

@@ -29,6 +29,8 @@ SIGNATURES = {
                           ci, ci, ci, cf, cf, ci],
     'tmx_swiglu': [vp, vp, vp, ci, vp, ci, ci, vp, ci, cf, vp, ci, ci],
     'tmx_qlora_gate_up_swiglu': [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cf],
+    'tmx_qlora_gate_up_swiglu_handover': [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cf],
+    'tmx_handover_status': [vp, vp],
     'tmx_gqa_decode_attention': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci],
     'tmx_gqa_attention_rows': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci, ci],
     'tmx_head_sample': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
@@ -51,6 +53,7 @@ SIZE_FUNCS = {
     'tmx_nucleus_workspace_bytes': [ci, ci],
     'tmx_qlora_linear_delta_workspace_bytes': [ci, ci, ci, ci, ci, ci],
     'tmx_decode_workspace_bytes': [vp, ci, ci],
+    'tmx_qlora_gate_up_swiglu_handover_bytes': [ci, ci, ci, ci],
 }
 
 

@@ -86,7 +86,8 @@ static Splits plan_splits(const tmx_model_desc* m, int B) {
 static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   Workspace w;
   size_t off = 0;
-  auto take = [&](size_t bytes) { char* p = base ? base + off : nullptr; off += align256(bytes); return p; };
+  // a region of zero bytes has no address: its pointer is null, and users test the pointer
+  auto take = [&](size_t bytes) { char* p = (base && bytes) ? base + off : nullptr; off += align256(bytes); return p; };
   const size_t D = m->embed_dim, NH = (size_t)m->num_heads * m->head_dim;
   const size_t QKV = NH + 2 * (size_t)m->num_kv_heads * m->head_dim, F = m->hidden_dim;
   const Splits sp = plan_splits(m, B);

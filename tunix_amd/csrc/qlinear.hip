@@ -1875,6 +1875,19 @@ size_t qlinear_gate_up_sync_bytes(int M, int K) {
   return 256 + (size_t)(K / 256) * mt * 4096 + mt * 32 * 64;
 }
 
+// The hand-over mode of the 8-wave kernel: t = x . A by K / 256 extra workgroups of the launch.  The main
+// workgroups wait (a bounded number of polls) for the producers, which sit first in dispatch order; the
+// launch is kept to one workgroup per compute unit of the device so that no main workgroup can hold a
+// unit a producer still needs.
+static bool gate_up_handover_shape(int M, int K, int F, int r) {
+  return M > 0 && M <= 64 && K % 512 == 0 && K < 8192 && F % 64 == 0 && r > 0 && 2 * r <= 32 && K / 256 <= 32 &&
+         F / 64 + K / 256 <= device_cus();
+}
+
+size_t qlinear_gate_up_handover_bytes(int M, int K, int F, int r) {
+  return gate_up_handover_shape(M, K, F, r) ? qlinear_gate_up_sync_bytes(M, K) : 0;
+}
+
 int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* qw, const void* scales,
                            const void* a_t, const void* lora_b, int r, float ls, void* act, int M, int K,
                            int F, int G, void* sync_ws, uint32_t* status) {
@@ -1907,10 +1920,8 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
   // up to 64 rows: 8 waves per workgroup, when steps of 8 k-tiles divide K and 32-bit byte
   // offsets reach every operand (128 rows would not fit the register file at 2 waves per SIMD)
   if (M <= 64 && K % 512 == 0 && (size_t)M * ldx * 2 < (1u << 31) && (size_t)K * F < (1u << 31)) {
-    if (a_t && sync_ws && K / 256 <= 32 && a.n_main_blocks + K / 256 <= 256) {
-      // t = x . A by K / 256 extra workgroups of the launch, handed to the others through memory; every
-      // workgroup must be resident at once (one per CU), or a main workgroup could wait for a producer
-      // that has no CU to run on
+    if (a_t && sync_ws && gate_up_handover_shape(M, K, F, r)) {
+      // t = x . A by K / 256 extra workgroups of the launch, handed to the others through memory
       const int mt = M <= 32 ? 1 : 2;
       a.sync = (uint32_t*)sync_ws;
       a.sync_status = status;
@@ -1955,7 +1966,7 @@ bool qlinear_delta_ok(int M, int K, int N, int Rpad, int r, int nsplit) {
   const int nls = qlinear_num_lora_splits(K, N);
   const int lbps = (nls + nsplit - 1) / nsplit;
   const int blocks = ((N + 127) / 128 + lbps) * nsplit;
-  if (blocks > (M > 64 ? 256 : 512) || (size_t)M * N * 2 >= (1u << 31)) return false;
+  if (blocks > device_cus() * (M > 64 ? 1 : 2) || (size_t)M * N * 2 >= (1u << 31)) return false;
   // The stage is a chain of round trips behind the LoRA blocks' own slices (arrive, wait, sum of the planes,
   // tiles: 6 to 10 us); it stays hidden only behind main blocks of at least 8 steps, and with at most two
   // column tiles per wave.  Shorter projections (measured: q|k|v and o of the 8B shape, 4 steps, 14.5 -> 21 us and
@@ -2156,6 +2167,24 @@ extern "C" int tmx_qlora_linear_planes(void* stream, const void* x, const void* 
                       TMX_MAX_RPAD, M, K, N, G, r_pad, nsplit);
 }
 
+// Word of a hand-over workspace (the first 256 bytes are its state block, cleared by the call) that a
+// kernel sets when its bounded wait ran out; tmx_handover_status reads it.
+static constexpr int kHandoverStatusWord = 63;
+
+extern "C" int tmx_handover_status(void* stream, void* workspace) {
+  if (!workspace) return TMX_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  uint32_t flag = 0;
+  uint32_t* word = (uint32_t*)workspace + kHandoverStatusWord;
+  if (hipMemcpyAsync(&flag, word, 4, hipMemcpyDeviceToHost, st) != hipSuccess) return TMX_ERR_LAUNCH;
+  if (hipStreamSynchronize(st) != hipSuccess) return TMX_ERR_LAUNCH;
+  if (flag == 0) return TMX_OK;
+  int rc = zero_words(st, word, 1);
+  if (rc != TMX_OK) return rc;
+  if (hipStreamSynchronize(st) != hipSuccess) return TMX_ERR_LAUNCH;
+  return TMX_ERR_DEVICE_WAIT;
+}
+
 extern "C" size_t tmx_qlora_linear_delta_workspace_bytes(int M, int K, int N, int r, int r_pad, int nsplit) {
   return qlinear_delta_ok(M, K, N, r_pad, r, nsplit) ? qlinear_delta_sync_bytes(M, r_pad) : 0;
 }
@@ -2170,6 +2199,7 @@ extern "C" int tmx_qlora_linear_planes_delta(void* stream, const void* x, const 
   ld.lora_b = (const uint16_t*)lora_b; ld.r = r; ld.ls = lora_scale;
   ld.seg_end[0] = seg_end0; ld.seg_end[1] = seg_end1; ld.seg_end[2] = N;
   ld.sync_ws = workspace;
+  ld.status = (uint32_t*)workspace + kHandoverStatusWord;
   int rc = zero_words((hipStream_t)stream, (uint32_t*)workspace, 64);
   if (rc != TMX_OK) return rc;
   return qlinear_base((hipStream_t)stream, x, K, qweight, scales, lora_a_t, nullptr, y_part, t_part, TMX_MAX_RPAD, M, K, N, G,
@@ -2247,6 +2277,21 @@ extern "C" int tmx_qlora_linear_noalloc(void* stream, const void* x, const void*
   // so nothing in the array has to start at zero
   return tmx_qlora_linear(stream, x, qweight, scales, lora_a_t, lora_b, residual, y, ws, M, K, N, G, r, r_pad,
                           lora_scale);
+}
+
+extern "C" size_t tmx_qlora_gate_up_swiglu_handover_bytes(int M, int K, int F, int r) {
+  return qlinear_gate_up_handover_bytes(M, K, F, r);
+}
+
+extern "C" int tmx_qlora_gate_up_swiglu_handover(void* stream, const void* x, const void* qweight, const void* scales,
+                                                 const void* lora_a_t, const void* lora_b, void* act, void* workspace,
+                                                 int M, int K, int F, int G, int r, float lora_scale) {
+  if (!lora_a_t || !lora_b || !workspace) return TMX_ERR_ARG;
+  if (qlinear_gate_up_handover_bytes(M, K, F, r) == 0) return TMX_ERR_UNSUPPORTED;
+  int rc = zero_words((hipStream_t)stream, (uint32_t*)workspace, 64);
+  if (rc != TMX_OK) return rc;
+  return qlinear_gate_up_swiglu((hipStream_t)stream, x, K, qweight, scales, lora_a_t, lora_b, r, lora_scale, act,
+                                M, K, F, G, workspace, (uint32_t*)workspace + kHandoverStatusWord);
 }
 
 extern "C" int tmx_qlora_gate_up_swiglu(void* stream, const void* x, const void* qweight, const void* scales,

@@ -291,6 +291,9 @@ int qlinear_gate_up_swiglu(hipStream_t st, const void* x, int ldx, const void* q
                            int F, int G, void* sync_ws, uint32_t* status = nullptr);
 size_t qlinear_gate_up_sync_bytes(int M, int K);
 int zero_words(hipStream_t st, uint32_t* p, int n);  // p[0 .. n) = 0 by a small kernel
+int device_cus();  // compute units of the current device (256 when none answers)
+// 0 when the fused gate | up launch cannot hand its LoRA projection over for this shape on this device
+size_t qlinear_gate_up_handover_bytes(int M, int K, int F, int r);
 // Many rows (M > 128), unsplit: y_bf16 = bf16(bf16(x . W) + bf16(bf16(t . B) ls)) in one pass, t = bf16(x . A)
 // computed by a LoRA-only launch of the same kernel and a small reduction (t_part: f32 planes, t16: bf16
 // [M][TMX_MAX_RPAD] scratch).  seg_end: column ends of the fused matrices (q | k | v, gate | up), unused
