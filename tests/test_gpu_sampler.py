@@ -34,15 +34,22 @@ def _sampler(model, cfg, cache_size):
   return Sampler(model, C.ToyTokenizer(), CacheConfig(cache_size, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
 
 
-def _compare_greedy(out, ref, n_rows, min_checked, lp_extra=0.0):
+def _compare_greedy(out, ref, n_rows, min_checked, lp_extra=0.0, logit_ulps=0):
+  """Tokens must agree wherever the oracle's top-2 margin exceeds the logit tolerance.  logit_ulps (needs
+  keep_logits): logits are bf16 values, so where they are large enough for a bf16 ulp to exceed the
+  tolerance, a last-bit flip of each of the two best logits is admitted on top of it."""
   margins = np.array(ref['state'].margins)  # [steps, B]
+  tol = np.full_like(margins, LOGIT_TOL)
+  if logit_ulps:
+    top = np.stack([z.max(-1) for z in ref['state'].step_logits])
+    tol = tol + logit_ulps * np.exp2(np.floor(np.log2(np.abs(top))) - 7)
   checked = 0
   for i in range(n_rows):
     got, want = out.tokens[i], ref['tokens'][i]
     assert len(got) == len(want)
     for s in range(len(want)):
       if got[s] != want[s]:
-        assert margins[s, i] <= LOGIT_TOL, (i, s, got[s], want[s], margins[s, i])
+        assert margins[s, i] <= tol[s, i], (i, s, got[s], want[s], margins[s, i], tol[s, i])
         break  # after a near-tie the two sequences legitimately differ
       assert abs(out.logprobs[i][s] - ref['logprobs'][i][s]) <= LOGPROB_TOL + lp_extra
       checked += 1
@@ -107,9 +114,10 @@ def test_wide_layer_at_33_to_64_sequences_matches_oracle(n_seq):
   cfg, oracle, s = _wide_pair()
   rng = np.random.default_rng(6 + n_seq)
   prompts = [rng.integers(3, cfg.vocab_size, 2 + i % 3) for i in range(n_seq)]
-  ref = OSAM.generate(oracle, cfg, prompts, 3, 16, eos_ids=(-1,))
+  ref = OSAM.generate(oracle, cfg, prompts, 3, 16, eos_ids=(-1,), keep_logits=True)
   out = s(prompt_token_ids=prompts, max_generation_steps=3, return_logprobs=True, eos_tokens=[-1])
-  _compare_greedy(out, ref, n_seq, 2 * n_seq, lp_extra=2.0 ** -5)
+  # 4096-wide hidden states against a 0.02-std head: the best logits lie in [4, 8), where one bf16 ulp is 2^-5
+  _compare_greedy(out, ref, n_seq, 3 * n_seq // 2, lp_extra=2.0 ** -5, logit_ulps=2)
   if n_seq == 64:
     _WIDE.clear()  # frees the device copy of the layer
 
