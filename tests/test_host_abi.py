@@ -4,6 +4,7 @@ input validation raises the reference's errors (tests/generate/sampler_test.py:1
 import ctypes
 import os
 import re
+import sys
 
 import numpy as np
 import pytest
@@ -325,3 +326,27 @@ def test_rollout_takes_the_actor_forms_the_cluster_hands_over(monkeypatch):
     TmxRollout._as_policy(Module(), 64, None, 7.5)
   with pytest.raises(TypeError, match='expected a QLoRAModel'):
     TmxRollout._as_policy(object(), 64, None, 7.5)
+
+
+def test_host_code_under_address_and_undefined_sanitizers():
+  """The host side of the C ABI (argument checks, slice planning, workspace carving: everything that runs
+  before the first launch) compiled with -fsanitize=address,undefined and driven over the shapes of the five
+  benchmark configurations in a child process that preloads the sanitizer runtime.  The sanitizer build is
+  made on first use and again when a source is newer than it (about two minutes; the device code is
+  compiled as usual, sanitizers apply to host code only)."""
+  import subprocess
+  from tunix_amd import build as tb
+  rt = tb.sanitizer_runtime()
+  if rt is None:
+    pytest.skip('clang AddressSanitizer runtime not found')
+  newest = max(os.path.getmtime(os.path.join(tb.CSRC, f)) for f in os.listdir(tb.CSRC))
+  newest = max(newest, os.path.getmtime(os.path.join(os.path.dirname(tb.CSRC), '..', 'include', 'tmx.h')))
+  if not os.path.exists(tb.HOSTSAN_LIB_PATH) or os.path.getmtime(tb.HOSTSAN_LIB_PATH) < newest:
+    tb.build(host_sanitizers=True)
+  env = dict(os.environ, TMX_LIB=tb.HOSTSAN_LIB_PATH, LD_PRELOAD=rt,
+             ASAN_OPTIONS='detect_leaks=0:abort_on_error=1', UBSAN_OPTIONS='halt_on_error=1:print_stacktrace=1')
+  child = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'host_sanitizer_child.py')
+  res = subprocess.run([sys.executable, child], capture_output=True, text=True, env=env, timeout=300)
+  assert res.returncode == 0, res.stdout + res.stderr
+  assert 'host sanitizer run ok' in res.stdout
+  assert 'AddressSanitizer' not in res.stderr and 'runtime error' not in res.stderr, res.stderr
