@@ -139,6 +139,8 @@ def main():
   ap.add_argument('--scoring', action='store_true',
                   help='time the scoring pass instead (Sampler.per_token_logps over prompt + new tokens of every '
                        'sequence): a separate JSON line, not the headline metric')
+  ap.add_argument('--no-kv-sharing', action='store_true',
+                  help='read the prompt slots per sequence even where consecutive rows hold samples of one prompt')
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--no-profile', action='store_true')
   ap.add_argument('--graph', action='store_true', help='replay one recorded decode step (tmx_decode_steps_graph)')
@@ -186,6 +188,7 @@ def main():
 
   sampler = Sampler(model, _Tok(), CacheConfig(cache_size, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
   sampler.eos_ids = np.array([-1])  # unreachable: every row runs the full length
+  sampler.share_prompt_kv = not args.no_kv_sharing
   rng = np.random.default_rng(0)
   # GRPO workloads: G = 8 samples of a prompt are consecutive rows; the others: distinct prompts
   n_prompts = max((batch + 7) // 8, 1) if 'grpo' in args.workload else batch

@@ -220,6 +220,21 @@ int tmx_gqa_decode_attention(void* stream, const void* q, const void* kcache, co
                              const uint8_t* input_mask, const int32_t* step, int buf_len, void* out,
                              void* workspace, int B, int N, int Kh, int H, int C);
 
+/* tmx_gqa_decode_attention for a batch made of consecutive groups of `share_group` sequences whose cache
+ * slots [0, share_len) hold identical K / V rows and identical input_mask entries: the G samples of one
+ * prompt that a GRPO rollout decodes side by side (tunix/rl/rl_learner.py:432-435 repeats every prompt
+ * num_generations times, in consecutive rows).  Those slots are read once per group, from the group's
+ * first sequence, for all of the group's queries; every sequence reads only its own slots from share_len
+ * on.  The softmax runs over the same positions as in tmx_gqa_decode_attention (the results differ in
+ * the order of the f32 sums only).  The caller vouches for the sharing; nothing checks that the rows
+ * really are equal.  B <= 128, B % share_group == 0, share_len >= 32, H in {64, 128}, N / Kh in
+ * {1, 2, 4}, else TMX_ERR_UNSUPPORTED.  workspace: tmx_gqa_decode_shared_workspace_bytes() bytes. */
+size_t tmx_gqa_decode_shared_workspace_bytes(int B, int N, int Kh, int H, int C);
+int tmx_gqa_decode_attention_shared(void* stream, const void* q, const void* kcache, const void* vcache,
+                                    const uint8_t* input_mask, const int32_t* step, int buf_len, void* out,
+                                    void* workspace, int B, int N, int Kh, int H, int C, int share_group,
+                                    int share_len);
+
 /* The same for T consecutive query tokens of every sequence (cache fill and scoring passes):
  * q and out are [n_seq * T, N H], row s * T + t is the token at slot *step + t of sequence s and
  * attends to the slots j <= *step + t with input_mask[s, j] (the causal mask of
@@ -352,6 +367,13 @@ typedef struct {
                               every projection has K % 128 == 0 (MoE models: rows * experts_per_tok <=
                               TMX_MAX_MOE_PAIRS), else 128.
                               The workspace must be sized for batch * T rows. */
+  int share_group;         /* 0 or 1: nothing is shared.  g > 1: the batch is made of consecutive groups of g
+                              sequences whose cache slots [0, share_len) and input_mask entries are identical
+                              (the samples of one prompt); one-token decode steps then read those slots once
+                              per group (see tmx_gqa_decode_attention_shared).  Ignored where the shared walk
+                              does not apply (more than 128 sequences, batch % g != 0, the 1..4-row path,
+                              tokens_per_pass > 1) */
+  int share_len;
 } tmx_decode_state;
 
 size_t tmx_decode_workspace_bytes(const tmx_model_desc* model, int batch, int cache_size);

@@ -378,6 +378,61 @@ def test_gqa_decode_attention(B, N, Kh, H, C, step):
   assert np.abs(got - ref).max() < 2e-2
 
 
+@pytest.mark.parametrize('B,N,Kh,H,C,step,gs,sl', [
+    (8, 8, 2, 64, 96, 70, 4, 32),        # two groups of four, one block of shared slots
+    (6, 4, 4, 128, 200, 150, 3, 64),     # one query head per kv head, groups of three
+    (16, 16, 8, 64, 300, 100, 16, 128),  # the step has not left the shared slots yet: they are walked up to it
+    (8, 32, 8, 128, 128, 63, 8, 64),     # first decode step after the prompt: no private slot yet
+    (12, 8, 2, 128, 400, 333, 6, 50),    # shared length that is no multiple of 32, two query blocks per group
+    (64, 32, 8, 128, 768, 520, 8, 256),  # the 8B rollout: 8 prompts x 8 samples at mid-generation
+    (64, 32, 8, 128, 768, 767, 8, 256),
+    (128, 32, 8, 128, 512, 300, 32, 224),  # four query blocks per group, one split of the shared slots
+])
+def test_gqa_decode_attention_with_shared_prompt_slots(B, N, Kh, H, C, step, gs, sl):
+  """tmx_gqa_decode_attention_shared: groups of gs sequences whose first sl cache slots and mask entries are
+  the same (the samples of one prompt, tunix/rl/rl_learner.py:432-435) against the oracle's attention of
+  every sequence over its own cache (tunix/models/llama3/model.py:379-396, mask of
+  tunix/generate/utils.py:35-59).  The shared slots of every sequence but a group's first are poisoned with
+  NaN in the device copy: the result stays finite, i.e. those rows are read once per group."""
+  T = G.Keep()
+  rng = np.random.default_rng(B * 1000 + C + gs)
+  q = bf16_round(rng.standard_normal((B, 1, N, H)).astype(np.float32))
+  k = bf16_round(rng.standard_normal((B, C, Kh, H)).astype(np.float32))
+  v = bf16_round(rng.standard_normal((B, C, Kh, H)).astype(np.float32))
+  in_mask = np.ones((B, C), bool)
+  lead = (np.arange(B) // gs) * gs
+  for b in range(B):
+    in_mask[b, : (lead[b] * 5 + 3) % max(min(step, sl) - 1, 1)] = False     # left padding, the same within a group
+    if step > sl + 8:
+      in_mask[b, sl + (b % 5)] = False                                      # and a private hole behind the prompt
+  in_mask[0, min(step, sl) // 2] = False
+  in_mask[:gs] &= in_mask[0]
+  in_mask[:, step] = True
+  k[:, :sl], v[:, :sl] = k[lead, :sl], v[lead, :sl]
+  in_mask[:, :sl] = in_mask[lead, :sl]
+  lib = _lib.lib()
+  ws = torch.empty(lib.tmx_gqa_decode_shared_workspace_bytes(B, N, Kh, H, C), dtype=torch.uint8, device=G.DEV)
+  out = torch.full((B, N * H), float('nan'), dtype=torch.bfloat16, device=G.DEV)
+  kd, vd = G.bf(k), G.bf(v)
+  follower = torch.from_numpy(np.arange(B) != lead).to(G.DEV)
+  kd[follower, :sl] = float('nan')
+  vd[follower, :sl] = float('nan')
+  G.call('tmx_gqa_decode_attention_shared', S(), T.bf(q), G.p(kd), G.p(vd), T.u8(in_mask), T.i32([step]), C,
+         G.p(out), G.p(ws), B, N, Kh, H, C, gs, sl)
+  G.sync()
+  from oracle import masks as OMK
+  mask = OMK.compute_attention_masks(step, C, ~in_mask)
+  fused = L.gqa_attention(q, k, v, mask, BF16, 'fused').reshape(B, -1)
+  ref = L.gqa_attention(q, k, v, mask, BF16, 'reference').reshape(B, -1)
+  got = G.host(out)
+  assert np.isfinite(got).all()
+  G.assert_bf16_close(got, fused, ulps=1.0, extra=1e-3, what='shared attention vs f32-internal oracle')
+  assert np.abs(got - ref).max() < 2e-2
+  # what the shared walk does not serve is refused, not silently run per row
+  assert lib.tmx_gqa_decode_attention_shared(S(), 1, 1, 1, 1, 1, 1, C, 1, 1, B, N, Kh, H, C, gs, 16) == -4
+  assert lib.tmx_gqa_decode_attention_shared(S(), 1, 1, 1, 1, 1, 1, C, 1, 1, B + 1, N, Kh, H, C, gs, sl) == -4
+
+
 @pytest.mark.parametrize('nseq,T,N,Kh,H,C,step', [
     (2, 40, 4, 4, 64, 64, 3), (3, 9, 8, 2, 64, 96, 50), (2, 33, 32, 8, 128, 300, 200), (1, 64, 8, 1, 128, 128, 0),
     (2, 5, 16, 8, 128, 96, 60), (1, 128, 4, 4, 128, 200, 31), (2, 3, 8, 4, 64, 64, 20),

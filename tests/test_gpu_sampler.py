@@ -195,6 +195,45 @@ def test_step_logits_within_tolerance_of_oracle():
     st['token_buffer'][:, 16 + step] = torch.from_numpy(tok).to(st['token_buffer'].device)
 
 
+def test_samples_of_one_prompt_share_its_cache_rows_and_match_oracle():
+  """Three prompts x four samples in consecutive rows (the GRPO layout, tunix/rl/rl_learner.py:432-435):
+  the Sampler finds the groups, decode attention reads the prompt slots once per group, and the per-step
+  logits and log-probs still match the oracle, which attends over every sequence's own cache.  Teacher
+  forcing with the oracle's SAMPLED tokens, so the rows of a group differ from the first generated token on."""
+  cfg = OM.Config('llama3', 2, 512, 256, 512, 8, 64, 2, norm_eps=1e-5)
+  oracle, model = _pair(cfg, seed=31, rank=8, alpha=16.0)
+  rng = np.random.default_rng(11)
+  base = [rng.integers(3, 512, n) for n in (70, 61, 66)]
+  prompts = [base[i // 4] for i in range(12)]
+  ref = OSAM.generate(oracle, cfg, prompts, 10, 96, eos_ids=(-1,), temperature=1.0, top_p=1.0, seed=5, keep_logits=True)
+  toks = ref['state'].token_buffer
+  ids = ref['padded_prompt_tokens']
+  p = ids.shape[1]  # the padded prompt length: the first generated token lands in column p
+  assert len({tuple(toks[i, p:p + 10]) for i in range(4)}) > 1   # the samples of a prompt do differ
+  runs = {}
+  for share in (True, False):
+    s = _sampler(model, cfg, 96)
+    s.share_prompt_kv = share
+    s.eos_ids = np.array([-1])
+    st = s.init_sample_state(ids, p + 10, True, None, 0.0, None, None, 0, include_logprobs=True,
+                             prompt_lengths=ref['prompt_lengths'])
+    assert (st['share_group'], st['share_len']) == ((4, p // 32 * 32) if share else (1, 0))
+    s.walk(st, p - 1)
+    steps = []
+    for step in range(10):
+      s.run_steps(st, 1, sample=True)
+      logits = st['logits'].cpu().numpy()
+      want = ref['state'].step_logits[step]
+      assert np.abs(logits - want).max() <= LOGIT_TOL, (share, step, np.abs(logits - want).max())
+      steps.append(logits)
+      tok = toks[:, p + step]
+      st['token_buffer'][:, p + step] = torch.from_numpy(tok).to(st['token_buffer'].device)
+    s.check_device_status(st)
+    runs[share] = np.stack(steps)
+  # shared and unshared walks: the same softmax over the same positions, only the order of the f32 sums differs
+  assert np.abs(runs[True] - runs[False]).max() <= 1e-2
+
+
 def test_temperature_sampling_follows_the_threefry_schedule():
   """Every generated token equals categorical(fold_in(PRNGKey(seed), decoding_step), logits / T)
   evaluated on the kernel's own logits, with decoding_step = P - 1, P, ... as in the reference

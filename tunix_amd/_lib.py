@@ -32,6 +32,7 @@ SIGNATURES = {
     'tmx_qlora_gate_up_swiglu_handover': [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cf],
     'tmx_handover_status': [vp, vp],
     'tmx_gqa_decode_attention': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci],
+    'tmx_gqa_decode_attention_shared': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci, ci, ci],
     'tmx_gqa_attention_rows': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci, ci],
     'tmx_head_sample': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
                         vp, vp],
@@ -47,6 +48,7 @@ SIGNATURES = {
 # entry points that return size_t
 SIZE_FUNCS = {
     'tmx_gqa_decode_workspace_bytes': [ci, ci, ci, ci, ci],
+    'tmx_gqa_decode_shared_workspace_bytes': [ci, ci, ci, ci, ci],
     'tmx_qlora_linear_workspace_bytes': [ci, ci, ci],
     'tmx_qlora_linear_noalloc_max_bytes': [],
     'tmx_head_sample_workspace_bytes': [ci, ci],

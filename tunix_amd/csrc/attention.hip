@@ -18,33 +18,48 @@
 
 namespace tmx {
 
+constexpr int kMaxPrefixSplits = 4;  // splits of the slots that a group of sequences shares
+
 // waves per workgroup: fewer for wide groups so the merge buffers stay under 64 KiB
 template <int G>
 struct AttnWaves { static constexpr int value = G > 4 ? 2 : 4; };
 
+// LDS of the one-token walk: merge buffers of the NG lane groups of a workgroup
 template <int H, int G>
-__global__ __launch_bounds__(AttnWaves<G>::value * 64, 4) void gqa_decode_kernel(AttnArgs a) {
+struct DecodeLds {
+  static constexpr int NW = AttnWaves<G>::value;
+  static constexpr int NG = NW * (64 / (H / 8));
+  float m[NG][G], l[NG][G];
+  float acc[NG][G][H];
+};
+
+template <int H, int G>
+__device__ __forceinline__ void gqa_decode_walk(const AttnArgs& a, DecodeLds<H, G>& lds, const int kvh, const int b,
+                                                const int split) {
   constexpr int NW = AttnWaves<G>::value;
   constexpr int LPP = H / 8;     // lanes per position row
   constexpr int PPW = 64 / LPP;  // positions per wave-wide load
   constexpr int U = 4;           // positions per lane group per iteration
   constexpr int NG = NW * PPW;   // lane groups per workgroup
-  __shared__ float s_m[NG][G], s_l[NG][G];
-  __shared__ float s_acc[NG][G][H];
+  auto& s_m = lds.m;
+  auto& s_l = lds.l;
+  auto& s_acc = lds.acc;
 
-  const int kvh = blockIdx.x, b = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int pg = lane / LPP, dl = lane % LPP;  // lane group, 8-element slice index
   const int tpp = a.tpp > 0 ? a.tpp : 1;
   const int seq = b / tpp;                    // b: query row of this pass
   // newest valid slot; clamped into the cache and the mask row so that a caller that oversteps reads in bounds
   const int step = min(*a.step + b % tpp, min(a.C, a.buf_len) - 1);
-  // the splits share the VALID positions 0 .. step (not the cache size) in chunks of whole
-  // 32 positions, so that every split has work at any context length
-  const int chunk = (((step + a.nsplit) / a.nsplit) + 31) & ~31;
-  const int s_begin = split * chunk;
+  // the splits share the VALID positions base .. step (not the cache size) in chunks of whole
+  // 32 positions, so that every split has work at any context length; base > 0: the slots below it
+  // are shared by a group of sequences and walked once per group by gqa_prefix_walk
+  const int base = a.share_gs > 1 ? min(a.share_len, step + 1) : 0;
+  const int chunk = (((step - base + a.nsplit) / a.nsplit) + 31) & ~31;
+  const int s_begin = base + split * chunk;
   int s_end = s_begin + chunk;
   if (s_end > step + 1) s_end = step + 1;
+  const int nparts = a.nsplit + a.psplits;  // partial results per row to be merged
 
   // query fragments for the G heads of this kv head: 8 bf16 = 4 packed pairs each
   uint32_t qf[G][4];
@@ -150,10 +165,10 @@ __global__ __launch_bounds__(AttnWaves<G>::value * 64, 4) void gqa_decode_kernel
       ls += s_l[i][g] * w;
       o += s_acc[i][g][d] * w;
     }
-    if (a.nsplit == 1) {
+    if (nparts == 1) {
       a.out[((size_t)b * a.N + kvh * G + g) * H + d] = f2bf(ls > 0.f ? o / ls : 0.f);
     } else {
-      float* pr = a.partial + ((((size_t)b * a.Kh + kvh) * a.nsplit + split) * G + g) * (H + 2);
+      float* pr = a.partial + ((((size_t)b * a.Kh + kvh) * nparts + split) * G + g) * (H + 2);
       pr[d] = o;
       if (d == 0) {
         pr[H] = mm;
@@ -164,19 +179,291 @@ __global__ __launch_bounds__(AttnWaves<G>::value * 64, 4) void gqa_decode_kernel
 }
 
 template <int H, int G>
+__global__ __launch_bounds__(AttnWaves<G>::value * 64, 4) void gqa_decode_kernel(AttnArgs a) {
+  __shared__ DecodeLds<H, G> lds;
+  gqa_decode_walk<H, G>(a, lds, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+template <int H, int G>
 __global__ __launch_bounds__(H) void gqa_combine_kernel(AttnArgs a) {
   const int kvh = blockIdx.x, b = blockIdx.y, g = blockIdx.z, d = threadIdx.x;
-  const float* pr = a.partial + (((size_t)b * a.Kh + kvh) * a.nsplit * G + g) * (H + 2);
+  const int nparts = a.nsplit + a.psplits;
+  const float* pr = a.partial + (((size_t)b * a.Kh + kvh) * nparts * G + g) * (H + 2);
   const size_t sstride = (size_t)G * (H + 2);
   float mm = -1e30f;
-  for (int s = 0; s < a.nsplit; ++s) mm = fmaxf(mm, pr[s * sstride + H]);
+  for (int s = 0; s < nparts; ++s) mm = fmaxf(mm, pr[s * sstride + H]);
   float ls = 0.f, o = 0.f;
-  for (int s = 0; s < a.nsplit; ++s) {
+  for (int s = 0; s < nparts; ++s) {
     const float w = __expf(pr[s * sstride + H] - mm);
     ls += pr[s * sstride + H + 1] * w;
     o += pr[s * sstride + d] * w;
   }
   a.out[((size_t)b * a.N + kvh * G + g) * H + d] = f2bf(ls > 0.f ? o / ls : 0.f);
+}
+
+// ---------------------------------------------------------------------------
+// Prompt slots shared by a group of sequences.  A GRPO rollout decodes G samples of every prompt as
+// consecutive rows (tunix/rl/rl_learner.py:432-435 repeats each prompt num_generations times), so the
+// K / V rows of the prompt slots are the same in the share_gs caches of a group, and so are their
+// input_mask entries.  The walk over those slots is then done once per (group, kv head) instead of once
+// per (sequence, kv head): the 32 / G sequences x G query heads of a query block are the 32 columns of
+// an MFMA tile, scores^T [position, query] = K . Q^T and out^T [hidden, query] += V^T . P^T exactly as in
+// the many-tokens kernel below, with the four waves of a workgroup taking different blocks of 32
+// positions.  K rows go from global memory straight into the A operand (lane (position, h) owns one half
+// of its row), the V tile of a wave goes global -> LDS by direct loads and is gathered transposed with
+// 16-bit reads, the query fragments wait in LDS.  Every row keeps its own slots share_len .. *step for
+// gqa_decode_walk, in the same launch (gqa_shared_kernel); both write (out, max, sum) partial results that
+// gqa_combine_kernel merges, so the attention of a row is the same softmax over the same positions as without
+// sharing (f32 throughout,
+// probabilities enter the V product as bf16 hi + lo).  The results differ from the unshared walk only in
+// the order of the f32 sums.
+
+template <int H>
+struct PrefixLds {
+  // the V tiles [4 waves][32 positions][H] bf16 are reused after the walk for the waves' accumulators
+  // [2][H / 32][16][64] f32 (two of the four waves at a time)
+  static constexpr int kTileBytes = 4 * 32 * H * 2;
+  static constexpr int kMergeBytes = 2 * (H / 32) * 16 * 64 * 4;
+  __attribute__((aligned(16))) unsigned char tiles[kTileBytes > kMergeBytes ? kTileBytes : kMergeBytes];
+  __attribute__((aligned(16))) uint16_t q[32 * H];  // query fragments [H / 8 chunks][32 queries][8]
+  float m[2][32], l[2][32];
+};
+
+template <int H, int G>
+__device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>& lds, const int kvh, const int gq,
+                                                const int ps) {
+  constexpr int KS = H / 16;        // MFMA k-steps of the score product
+  constexpr int CPR = H / 8;        // 16-byte chunks per cache row
+  constexpr int RPD = 64 / CPR;     // rows per 1 KiB direct-to-LDS load
+  constexpr int NLD = 32 / RPD;     // loads per wave and V tile
+  constexpr int HT = H / 32;        // hidden tiles of the output
+  constexpr int RPB = 32 / G;       // sequences per query block
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int h = lane >> 5, qi = lane & 31;
+  const int qblocks = (a.share_gs + RPB - 1) / RPB;
+  const int grp = gq / qblocks, qb = gq - grp * qblocks;
+  const int lead = grp * a.share_gs;  // the group's first sequence: its cache rows and mask are the ones read
+  const int step = min(*a.step, min(a.C, a.buf_len) - 1);
+  const int plen = min(a.share_len, step + 1);
+  const int nblk = (plen + 31) >> 5;
+  const int bps = (nblk + a.psplits - 1) / a.psplits;
+  const int b_end = min((ps + 1) * bps, nblk);
+
+  // query fragments of the block into LDS: thread (query, chunk) copies 16 bytes; rows past the group
+  // repeat its last sequence (their results are not stored)
+  for (int e = threadIdx.x; e < 32 * CPR; e += 256) {
+    const int q = e / CPR, c = e % CPR;
+    const int lr = min(qb * RPB + q / G, a.share_gs - 1);
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)(lead + lr) * a.N + kvh * G + q % G) * H + c * 8);
+    *reinterpret_cast<u32x4_t*>(lds.q + (c * 32 + q) * 8) = v;
+  }
+  __syncthreads();
+
+  const uint32_t row_bytes = (uint32_t)a.Kh * H * 2;
+  const uint32_t span = ((uint32_t)(a.C - 1) * a.Kh + 1) * H * 2;  // rows past the cache read zero
+  const __amdgpu_buffer_rsrc_t rk = make_rsrc(a.kcache + ((size_t)lead * a.C * a.Kh + kvh) * H, span);
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(a.vcache + ((size_t)lead * a.C * a.Kh + kvh) * H, span);
+  uint16_t* vt = reinterpret_cast<uint16_t*>(lds.tiles) + wave * 32 * H;
+  // V tile transfer: load i moves rows i RPD .. i RPD + RPD - 1 of the block, the 16-byte chunks of row r
+  // XOR-swizzled by r % CPR.  Row i RPD + lane / CPR has r % CPR = (i RPD) % CPR ^ lane / CPR, so the per-lane
+  // part of the swizzle is one word and the rest a constant per load; the offsets are formed at the transfer
+  // (kept in registers over the loop they would be spilled)
+  const int vrow = (lane / CPR) * row_bytes, vswz = (lane % CPR) ^ (lane / CPR);
+  auto dma_v = [&](int blk) __attribute__((always_inline)) {
+    int sw = vswz;
+    asm volatile("" : "+v"(sw));
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      load_row_to_lds(rv, vt + i * RPD * H, vrow + ((sw ^ ((i * RPD) % CPR)) << 4), (blk * 32 + i * RPD) * row_bytes);
+  };
+  // K fragments of a block: lane (position qi, h) reads the half h of its row, 16 bytes per MFMA step
+  const int koff = qi * row_bytes + h * H;
+  u32x4_t kf[KS];
+  auto load_k = [&](int blk) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < KS; ++t)
+      kf[t] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rk, koff + t * 16, blk * 32 * row_bytes, 0));
+  };
+  const uint8_t* mrow = a.input_mask + (size_t)lead * a.buf_len;
+  auto mask_byte = [&](int blk) __attribute__((always_inline)) {
+    const int p = blk * 32 + qi;
+    return (h == 0 && p < a.buf_len) ? mrow[p] : (uint8_t)0;
+  };
+
+  f32x16_t o[HT];
+#pragma unroll
+  for (int c = 0; c < HT; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[c][r] = 0.f;
+  float m = -1e30f, l = 0.f;
+
+  int blk = ps * bps + wave;
+  uint8_t mb = 0;
+  if (blk < b_end) {
+    mb = mask_byte(blk);
+    load_k(blk);
+    dma_v(blk);
+  }
+  for (; blk < b_end; blk += 4) {
+    const bool more = blk + 4 < b_end;
+    const uint32_t mbits = (uint32_t)__ballot(mb != 0);
+    // scores^T: rows = positions of the block, column = this lane's query
+    f32x16_t sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+    for (int t = 0; t < KS; ++t) {
+      const bf16x8_t qf = *reinterpret_cast<const bf16x8_t*>(lds.q + ((KS * h + t) * 32 + qi) * 8);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf[t]), qf, sacc, 0, 0, 0);
+    }
+    float sc[16];
+    float mn = m;
+    // accumulator register r holds position 8 (r / 4) + 4 h + r % 4 of the block: with the lane's half folded
+    // into the mask word and the limit, the per-register part is a compile-time constant
+    const uint32_t mb2 = mbits >> (4 * h);
+    const int lim = plen - blk * 32 - 4 * h;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int pc = (r >> 2) * 8 + (r & 3);
+      const bool ok = pc < lim && ((mb2 >> pc) & 1u);
+      sc[r] = ok ? sacc[r] * a.scale : -1e30f;
+      mn = fmaxf(mn, sc[r]);
+    }
+    mn = fmaxf(mn, __shfl_xor(mn, 32, 64));
+    const float alpha = __expf(m - mn);
+    m = mn;
+    float psum = 0.f;
+    uint32_t pk[8], pl2[8];
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      const float p0 = sc[r] > -1e29f ? __expf(sc[r] - mn) : 0.f;
+      const float p1 = sc[r + 1] > -1e29f ? __expf(sc[r + 1] - mn) : 0.f;
+      pk[r >> 1] = pack_bf2(p0, p1);
+      pl2[r >> 1] = pack_bf2(p0 - bf_lo(pk[r >> 1]), p1 - bf_hi(pk[r >> 1]));
+      psum += p0 + p1;
+    }
+    l = l * alpha + psum;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int c = 0; c < HT; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[c][r] *= alpha;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this block's V tile has landed
+    // out^T += V^T . P^T, 16 positions (accumulator registers 8 kb .. 8 kb + 7) per MFMA.  The V^T fragment is
+    // gathered with 16-bit reads: element (row, hidden 32 c + qi) of the tile, row = acc_row(8 kb + j, lane) =
+    // 8 (2 kb + j / 4) + 4 h + j % 4, sits in chunk (4 c + qi / 8) ^ row % CPR; the lane's share of that XOR is
+    // one word (gsw), the rest a constant per read, and the addresses are formed here, read by read
+    {
+      int gsw = (qi >> 3) ^ ((4 * h) % CPR), gbase = 4 * h * H + (qi & 7);
+      asm volatile("" : "+v"(gsw), "+v"(gbase));
+#pragma unroll
+      for (int kb2 = 0; kb2 < 2; ++kb2) {
+        const u32x4_t pf = {pk[4 * kb2], pk[4 * kb2 + 1], pk[4 * kb2 + 2], pk[4 * kb2 + 3]};
+        const u32x4_t pg = {pl2[4 * kb2], pl2[4 * kb2 + 1], pl2[4 * kb2 + 2], pl2[4 * kb2 + 3]};
+#pragma unroll
+        for (int c = 0; c < HT; ++c) {
+          uint32_t vw[4];
+#pragma unroll
+          for (int j2 = 0; j2 < 4; ++j2) {
+            uint32_t e2[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const int j = 2 * j2 + e;
+              const int row0 = (2 * kb2 + j / 4) * 8 + (j & 3);  // the row without the lane's 4 h
+              e2[e] = vt[gbase + row0 * H + ((gsw ^ (4 * c) ^ (row0 % CPR)) << 3)];
+            }
+            vw[j2] = e2[0] | (e2[1] << 16);
+          }
+          const u32x4_t vf = {vw[0], vw[1], vw[2], vw[3]};
+          o[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                         __builtin_bit_cast(bf16x8_t, pf), o[c], 0, 0, 0);
+          o[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                         __builtin_bit_cast(bf16x8_t, pg), o[c], 0, 0, 0);
+        }
+      }
+    }
+    // the tile's reads are complete before the next transfer overwrites it.  The next block's K rows are
+    // requested only now (not under the softmax): 32 more live registers would not fit three workgroups per CU,
+    // and the other eleven waves of the CU cover the round trip.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (more) {
+      mb = mask_byte(blk + 4);
+      load_k(blk + 4);
+      dma_v(blk + 4);
+    }
+  }
+  l += __shfl_xor(l, 32, 64);
+
+  // merge the four waves in two rounds through LDS: waves 2, 3 hand their state to waves 0, 1, then wave 1 to
+  // wave 0.  The accumulator layout is the same in every wave, so the merge is per lane.
+  float* mb_f = reinterpret_cast<float*>(lds.tiles);
+  auto put = [&](int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int c = 0; c < HT; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mb_f[(((slot * HT + c) * 16 + r) << 6) + lane] = o[c][r];
+    if (h == 0) {
+      lds.m[slot][qi] = m;
+      lds.l[slot][qi] = l;
+    }
+  };
+  auto take = [&](int slot) __attribute__((always_inline)) {
+    const float m2 = lds.m[slot][qi], l2 = lds.l[slot][qi];
+    const float mm = fmaxf(m, m2);
+    const float w1 = __expf(m - mm), w2 = __expf(m2 - mm);
+#pragma unroll
+    for (int c = 0; c < HT; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[c][r] = o[c][r] * w1 + mb_f[(((slot * HT + c) * 16 + r) << 6) + lane] * w2;
+    l = l * w1 + l2 * w2;
+    m = mm;
+  };
+  __syncthreads();  // every wave is done with its V tile
+  if (wave >= 2) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) take(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave != 0) return;
+  take(0);
+  // wave 0 holds out^T [hidden, query] for the block's queries: one part per (sequence, query head)
+  const int lr = qb * RPB + qi / G, g = qi % G;
+  if (lr >= a.share_gs) return;
+  const int nparts = a.nsplit + a.psplits;
+  float* pr = a.partial + ((((size_t)(lead + lr) * a.Kh + kvh) * nparts + a.nsplit + ps) * G + g) * (H + 2);
+#pragma unroll
+  for (int c = 0; c < HT; ++c)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // accumulator registers 4 i .. 4 i + 3 of tile c: hidden values 32 c + 8 i + 4 h .. + 3 (a part is H + 2
+      // floats: 8-byte aligned pieces)
+      float* d = pr + 32 * c + 8 * i + 4 * h;
+      *reinterpret_cast<f32x2_t*>(d) = f32x2_t{o[c][4 * i], o[c][4 * i + 1]};
+      *reinterpret_cast<f32x2_t*>(d + 2) = f32x2_t{o[c][4 * i + 2], o[c][4 * i + 3]};
+    }
+  if (h == 0) {
+    pr[H] = m;
+    pr[H + 1] = l;
+  }
+}
+
+// One launch for both walks: blockIdx.y below n_prefix_y = (group, query block) of the shared slots, the rest one
+// row each (the groups' workgroups first in dispatch order).  Three workgroups per CU (LDS and registers), so
+// that the rows' workgroups and the groups' are all resident at a rollout's batch sizes.
+template <int H, int G>
+__global__ __launch_bounds__(256, 3) void gqa_shared_kernel(AttnArgs a, int n_prefix_y) {
+  union Lds {
+    DecodeLds<H, G> d;
+    PrefixLds<H> p;
+  };
+  __shared__ Lds lds;
+  if ((int)blockIdx.y < n_prefix_y) {
+    if ((int)blockIdx.z < a.psplits) gqa_prefix_walk<H, G>(a, lds.p, blockIdx.x, blockIdx.y, blockIdx.z);
+    return;
+  }
+  if ((int)blockIdx.z < a.nsplit) gqa_decode_walk<H, G>(a, lds.d, blockIdx.x, (int)blockIdx.y - n_prefix_y, blockIdx.z);
 }
 
 // ---------------------------------------------------------------------------
@@ -383,11 +670,62 @@ size_t attn_partial_bytes(int B, int N, int Kh, int H, int C) {
   return ns == 1 ? 0 : (size_t)B * N * ns * (H + 2) * sizeof(float);
 }
 
+// Splits of the shared slots: two waves of a workgroup get one block of 32 positions each, up to
+// kMaxPrefixSplits workgroups per (group, kv head, query block) (measured on 256 shared slots at 64 sequences:
+// 1, 2, 4 splits -> 23.9, 22.1, 21.2 us for the launch; the combine launch behind it reads one more part per split).
+static int prefix_splits(int share_len) {
+  const int nblk = (share_len + 31) / 32;
+  int ps = nblk / 2;
+  if (ps < 1) ps = 1;
+  return ps > kMaxPrefixSplits ? kMaxPrefixSplits : ps;
+}
+
+size_t attn_shared_partial_bytes(int B, int N, int Kh, int H, int C) {
+  return (size_t)B * N * (attn_num_splits(B, Kh, C) + kMaxPrefixSplits) * (H + 2) * sizeof(float);
+}
+
+// The shared walk serves one token per sequence, up to 128 sequences in whole groups, head dimensions and
+// group widths of the MFMA tile (G query heads per kv head, G in {1, 2, 4}), and 32-bit byte offsets per cache.
+bool attn_share_ok(int B, int N, int Kh, int H, int C, int share_gs, int share_len) {
+  if (share_gs <= 1 || share_len < 32 || share_len > C || B <= 0 || B > 128 || B % share_gs) return false;
+  if (Kh <= 0 || N % Kh || (H != 64 && H != 128)) return false;
+  const int G = N / Kh;
+  if (G != 1 && G != 2 && G != 4) return false;
+  return (size_t)C * Kh * H * 2 < (1u << 31);
+}
+
+template <int H, int G>
+static int launch_shared(hipStream_t st, const AttnArgs& a) {
+  const int rpb = 32 / G, qblocks = (a.share_gs + rpb - 1) / rpb;
+  const int n_prefix_y = (a.B / a.share_gs) * qblocks;
+  const int nz = a.nsplit > a.psplits ? a.nsplit : a.psplits;
+  hipLaunchKernelGGL((gqa_shared_kernel<H, G>), dim3(a.Kh, n_prefix_y + a.B, nz), dim3(256), 0, st, a, n_prefix_y);
+  int rc = check_launch();
+  if (rc != TMX_OK) return rc;
+  hipLaunchKernelGGL((gqa_combine_kernel<H, G>), dim3(a.Kh, a.B, G), dim3(H), 0, st, a);
+  return check_launch();
+}
+
 int gqa_decode(hipStream_t st, AttnArgs a, int H) {
   a.nsplit = attn_num_splits(a.B, a.Kh, a.C);
-  if (a.nsplit > 1 && !a.partial) return TMX_ERR_ARG;
   const int G = a.N / a.Kh;
   if (a.N % a.Kh) return TMX_ERR_SHAPE;
+  if (a.tpp <= 1 && attn_share_ok(a.B, a.N, a.Kh, H, a.C, a.share_gs, a.share_len)) {
+    // G samples of a prompt in consecutive rows: the prompt slots once per group, the rest per row
+    if (!a.partial) return TMX_ERR_ARG;
+    a.psplits = prefix_splits(a.share_len);
+#define TMX_SHARED_CASE(HH, GG) \
+  if (H == HH && G == GG) return launch_shared<HH, GG>(st, a);
+    TMX_SHARED_CASE(64, 1)
+    TMX_SHARED_CASE(64, 2)
+    TMX_SHARED_CASE(64, 4)
+    TMX_SHARED_CASE(128, 1)
+    TMX_SHARED_CASE(128, 2)
+    TMX_SHARED_CASE(128, 4)
+#undef TMX_SHARED_CASE
+  }
+  a.share_gs = a.share_len = a.psplits = 0;
+  if (a.nsplit > 1 && !a.partial) return TMX_ERR_ARG;
   // several tokens per sequence: one walk over the cache for a block of them (MFMA kernel)
   if (a.tpp >= kFillMinTokens && a.B % a.tpp == 0 && (size_t)a.C * a.Kh * H * 2 < (1u << 31)) {
 #define TMX_FILL_CASE(HH, GG) \
@@ -438,6 +776,32 @@ extern "C" int tmx_gqa_decode_attention(void* stream, const void* q, const void*
   a.out = (uint16_t*)out;
   a.partial = (float*)workspace;
   a.B = B; a.N = N; a.Kh = Kh; a.C = C;
+  a.scale = 1.0f / sqrtf((float)H);
+  return gqa_decode((hipStream_t)stream, a, H);
+}
+
+extern "C" size_t tmx_gqa_decode_shared_workspace_bytes(int B, int N, int Kh, int H, int C) {
+  return attn_shared_partial_bytes(B, N, Kh, H, C);
+}
+
+extern "C" int tmx_gqa_decode_attention_shared(void* stream, const void* q, const void* kcache, const void* vcache,
+                                               const uint8_t* input_mask, const int32_t* step, int buf_len,
+                                               void* out, void* workspace, int B, int N, int Kh, int H, int C,
+                                               int share_group, int share_len) {
+  if (!q || !kcache || !vcache || !input_mask || !step || !out || !workspace) return TMX_ERR_ARG;
+  if (B <= 0 || N <= 0 || Kh <= 0 || C <= 0) return TMX_ERR_SHAPE;
+  if (!attn_share_ok(B, N, Kh, H, C, share_group, share_len)) return TMX_ERR_UNSUPPORTED;
+  AttnArgs a = {};
+  a.q = (const uint16_t*)q;
+  a.kcache = (const uint16_t*)kcache;
+  a.vcache = (const uint16_t*)vcache;
+  a.input_mask = input_mask;
+  a.step = step;
+  a.buf_len = buf_len;
+  a.out = (uint16_t*)out;
+  a.partial = (float*)workspace;
+  a.B = B; a.N = N; a.Kh = Kh; a.C = C;
+  a.share_gs = share_group; a.share_len = share_len;
   a.scale = 1.0f / sqrtf((float)H);
   return gqa_decode((hipStream_t)stream, a, H);
 }

@@ -114,7 +114,15 @@ static Workspace carve(const tmx_model_desc* m, int B, int C, char* base) {
   w.sb_tparts = (float*)take(small ? (F / 32 + 1) * (size_t)B * 32 * 4 : 0);
   w.sb_attn_partial = (float*)take(small ? sb_attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C) : 0);
   w.rope_tab = (float*)take((size_t)B * m->head_dim * 4);
-  w.attn_partial = (float*)take(attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C));
+  {
+    // split results of decode attention; up to 128 rows also room for the shared walk over prompt slots
+    size_t ab = attn_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C);
+    if (B <= 128) {
+      const size_t sb = attn_shared_partial_bytes(B, m->num_heads, m->num_kv_heads, m->head_dim, C);
+      if (sb > ab) ab = sb;
+    }
+    w.attn_partial = (float*)take(ab);
+  }
   w.head_partial = take(head_partial_bytes(B, m->vocab_size));
   const size_t P = m->num_experts > 0 ? (size_t)B * m->experts_per_tok : 0;
   w.expert_of = (int32_t*)take(P * 4);
@@ -247,6 +255,8 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
     rc = zero_words(st, (uint32_t*)w.gu_sync, 64);
     if (rc != TMX_OK) return rc;
   }
+  // samples of one prompt in consecutive rows: decode attention reads the prompt slots once per group
+  const bool share_walk = T == 1 && !small && w.attn_partial && attn_share_ok(B, N, Kh, H, C, s->share_group, s->share_len);
   for (int it = 0; it < n_steps; ++it) {
     {  // embedding gather + first input norm + this step's RoPE table
       RowNormArgs a = {};
@@ -379,6 +389,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         a.out = w.attn; a.partial = w.attn_partial;
         a.B = B; a.N = N; a.Kh = Kh; a.C = C;
         a.scale = 1.0f / sqrtf((float)H);
+        if (share_walk) { a.share_gs = s->share_group; a.share_len = s->share_len; }
         TMX_TRY(TMX_K_ATTN, gqa_decode(st, a, H));
       }
       {

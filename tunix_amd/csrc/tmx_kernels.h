@@ -162,6 +162,12 @@ struct AttnArgs {
   int B, N, Kh, C, nsplit, chunk;
   float scale;
   int tpp;  // tokens per pass (0: 1): query row m belongs to sequence m / tpp and sees slots <= *step + m % tpp
+  // Shared prompt slots (G samples of one prompt in consecutive rows): share_gs > 1 says that the sequences
+  // come in consecutive groups of share_gs whose cache slots [0, share_len) and input_mask entries are
+  // identical.  Those slots are then walked once per group (gqa_prefix_kernel, psplits splits, from the
+  // group's first sequence), every row walks only its own slots share_len .. *step (nsplit splits), and
+  // the nsplit + psplits partial results per row are merged by the rows' walk itself or the combine kernel.
+  int share_gs, share_len, psplits;
 };
 
 struct HeadArgs {
@@ -270,6 +276,9 @@ int advance_step(hipStream_t st, int32_t* step, int by);
 int empty_launch(hipStream_t st);  // measurement aid: a kernel that does nothing
 int gqa_decode(hipStream_t st, AttnArgs a, int H);
 size_t attn_partial_bytes(int B, int N, int Kh, int H, int C);
+// the same when the rows may share prompt slots (AttnArgs::share_gs > 1): room for the prefix partials too
+size_t attn_shared_partial_bytes(int B, int N, int Kh, int H, int C);
+bool attn_share_ok(int B, int N, int Kh, int H, int C, int share_gs, int share_len);
 int moe_route(hipStream_t st, const RouterArgs& a, int B);
 int moe_experts(hipStream_t st, const MoeArgs& a, int E, bool down);
 int head_sample(hipStream_t st, HeadArgs a);

@@ -105,7 +105,8 @@ class DecodeState(ctypes.Structure):
               ('n_eos', ctypes.c_int), ('forbidden', ctypes.c_void_p), ('n_forbidden', ctypes.c_int),
               ('logits_out', ctypes.c_void_p), ('workspace', ctypes.c_void_p),
               ('workspace_bytes', ctypes.c_size_t), ('nucleus_workspace', ctypes.c_void_p),
-              ('nucleus_workspace_bytes', ctypes.c_size_t), ('tokens_per_pass', ctypes.c_int)]
+              ('nucleus_workspace_bytes', ctypes.c_size_t), ('tokens_per_pass', ctypes.c_int),
+              ('share_group', ctypes.c_int), ('share_len', ctypes.c_int)]
 
 
 def _qdesc(pl):

@@ -76,6 +76,29 @@ def _seed_key(seed):
   return int(arr[0]), int(arr[1])
 
 
+def shared_prompt_groups(ids, mask, min_len=32, max_group=64):
+  """(g, n): the largest saving split of the rows into consecutive groups of g whose first n columns agree
+  in token ids and mask; (1, 0) when nothing is worth sharing.  A GRPO rollout decodes the G samples of a
+  prompt as consecutive rows (tunix/rl/rl_learner.py:432-435 repeats every prompt num_generations times), so
+  the K / V rows of the prompt columns are the same within a group and decode attention can read them once
+  per group.  n is rounded down to a multiple of 32; the saving counted is (g - 1) / g * n cache rows."""
+  ids, mask = np.asarray(ids), np.asarray(mask)
+  b, p = ids.shape
+  if b < 2 or p < min_len:
+    return 1, 0
+  same = (ids[1:] == ids[:-1]) & (mask[1:] == mask[:-1])          # row i + 1 against row i, per column
+  run = np.where(same.all(axis=1), p, np.argmin(same, axis=1))   # columns in which row i + 1 repeats row i
+  best, best_gain = (1, 0), 0.0
+  for g in range(2, min(b, max_group) + 1):
+    if b % g:
+      continue
+    inner = np.arange(1, b) % g != 0                              # pairs (i, i + 1) inside one group
+    n = int(run[inner[: b - 1]].min()) // 32 * 32
+    if n >= min_len and (g - 1) / g * n > best_gain:
+      best, best_gain = (g, n), (g - 1) / g * n
+  return best
+
+
 class Sampler:
   """Sampler for an int4 QLoRA decoder resident on one MI355X."""
 
@@ -99,6 +122,8 @@ class Sampler:
     # replay one recorded decode step instead of launching every kernel: measured neutral on
     # MI355X (the steps are bound by the device, not by host launches), so off by default
     self.use_graph = False
+    # read the cache rows of prompt columns once per group of rows with the same prompt (GRPO samples)
+    self.share_prompt_kv = True
     self.eos_ids = None
     self.last_step_logits = None
 
@@ -179,6 +204,7 @@ class Sampler:
     else:
       input_mask[:, :p] = ids != pad
     positions = utils.build_positions_from_mask(input_mask)
+    share = shared_prompt_groups(ids, input_mask[:, :p]) if self.share_prompt_kv else (1, 0)
     c = self._transformer.config
     need = (c.num_layers, 2, b, self.cache_config.cache_size, c.num_kv_heads, c.head_dim)
     if self._cache is None or tuple(self._cache.shape) != need:
@@ -198,6 +224,7 @@ class Sampler:
         'step': torch.zeros(1, dtype=torch.int32, device=dev),
         'cache': self._cache,
         'num_input_tokens': p,
+        'share_group': share[0], 'share_len': share[1],
         'total_sampling_steps': total_sampling_steps,
         'sampling_mode': 'greedy' if top_p is None else 'top_p',
         'temperature': float(temperature),
@@ -224,6 +251,7 @@ class Sampler:
       self._workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=self._transformer.device)
     s = DecodeState()
     s.tokens_per_pass = tokens_per_pass
+    s.share_group, s.share_len = st.get('share_group', 1), st.get('share_len', 0)
     s.batch, s.buf_len, s.cache_size = b, total, self.cache_config.cache_size
     s.token_buffer, s.positions = st['token_buffer'].data_ptr(), st['positions'].data_ptr()
     s.input_mask, s.done, s.step = st['input_mask'].data_ptr(), st['done'].data_ptr(), st['step'].data_ptr()
