@@ -116,8 +116,10 @@ def test_wide_layer_at_33_to_64_sequences_matches_oracle(n_seq):
   prompts = [rng.integers(3, cfg.vocab_size, 2 + i % 3) for i in range(n_seq)]
   ref = OSAM.generate(oracle, cfg, prompts, 3, 16, eos_ids=(-1,), keep_logits=True)
   out = s(prompt_token_ids=prompts, max_generation_steps=3, return_logprobs=True, eos_tokens=[-1])
-  # 4096-wide hidden states against a 0.02-std head: the best logits lie in [4, 8), where one bf16 ulp is 2^-5
-  _compare_greedy(out, ref, n_seq, 3 * n_seq // 2, lp_extra=2.0 ** -5, logit_ulps=2)
+  # 4096-wide hidden states against a 0.02-std head: the best logits lie in [4, 8), where one bf16 ulp is 2^-5.
+  # log-prob = chosen logit - logsumexp: a last-bit flip of the chosen logit moves it by one such ulp, flips of the
+  # few large logits that carry the log-sum-exp by up to another
+  _compare_greedy(out, ref, n_seq, 3 * n_seq // 2, lp_extra=2.0 ** -4, logit_ulps=2)
   if n_seq == 64:
     _WIDE.clear()  # frees the device copy of the layer
 

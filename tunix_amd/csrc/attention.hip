@@ -53,7 +53,7 @@ __device__ __forceinline__ void gqa_decode_walk(const AttnArgs& a, DecodeLds<H, 
   const int step = min(*a.step + b % tpp, min(a.C, a.buf_len) - 1);
   // the splits share the VALID positions base .. step (not the cache size) in chunks of whole
   // 32 positions, so that every split has work at any context length; base > 0: the slots below it
-  // are shared by a group of sequences and walked once per group by gqa_prefix_walk
+  // are shared by a group of sequences and walked once per group by the tile walk (gqa_shared_kernel)
   const int base = a.share_gs > 1 ? min(a.share_len, step + 1) : 0;
   const int chunk = (((step - base + a.nsplit) / a.nsplit) + 31) & ~31;
   const int s_begin = base + split * chunk;
@@ -202,21 +202,26 @@ __global__ __launch_bounds__(H) void gqa_combine_kernel(AttnArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Prompt slots shared by a group of sequences.  A GRPO rollout decodes G samples of every prompt as
-// consecutive rows (tunix/rl/rl_learner.py:432-435 repeats each prompt num_generations times), so the
-// K / V rows of the prompt slots are the same in the share_gs caches of a group, and so are their
-// input_mask entries.  The walk over those slots is then done once per (group, kv head) instead of once
-// per (sequence, kv head): the 32 / G sequences x G query heads of a query block are the 32 columns of
-// an MFMA tile, scores^T [position, query] = K . Q^T and out^T [hidden, query] += V^T . P^T exactly as in
-// the many-tokens kernel below, with the four waves of a workgroup taking different blocks of 32
-// positions.  K rows go from global memory straight into the A operand (lane (position, h) owns one half
-// of its row), the V tile of a wave goes global -> LDS by direct loads and is gathered transposed with
-// 16-bit reads, the query fragments wait in LDS.  Every row keeps its own slots share_len .. *step for
-// gqa_decode_walk, in the same launch (gqa_shared_kernel); both write (out, max, sum) partial results that
-// gqa_combine_kernel merges, so the attention of a row is the same softmax over the same positions as without
-// sharing (f32 throughout,
-// probabilities enter the V product as bf16 hi + lo).  The results differ from the unshared walk only in
-// the order of the f32 sums.
+// The one-token walk on the matrix pipe (gqa_tile_kernel).  The queries of a workgroup are the 32 columns of an
+// MFMA tile: scores^T [position, query] = K . Q^T and out^T [hidden, query] += V^T . P^T as in the many-tokens
+// kernel below, with the four waves of a workgroup taking different blocks of 32 positions and meeting through
+// LDS at the end.  K rows go from global memory straight into the A operand (lane (position, h) owns one half
+// of its row), the V tile of a wave goes global -> LDS by direct loads and is gathered transposed with 16-bit
+// reads, the query fragments wait in LDS.  Per 32 positions a wave issues 8 + 32 MFMAs and about 150 VALU
+// instructions, against about 1400 VALU instructions per 16 positions of gqa_decode_walk, whose dot products
+// and reductions run on the vector ALU; it takes the launch wherever its workgroups (three per CU: LDS and
+// registers) are all resident at once.
+//
+// Two kinds of query block share the launch:
+//  * a row: the G query heads of one sequence (the first G columns of the tile) over that sequence's own slots;
+//  * a group: prompt slots shared by a group of sequences.  A GRPO rollout decodes the samples of every prompt
+//    as consecutive rows (tunix/rl/rl_learner.py:432-435 repeats each prompt num_generations times), so the
+//    K / V rows of the prompt slots are the same in the share_gs caches of a group, and so are their input_mask
+//    entries.  Those slots are walked once per (group, kv head), from the group's first sequence, for the
+//    32 / G sequences x G query heads of a query block; every row keeps its own slots share_len .. *step.
+// A query block with one split writes its output directly; otherwise every walk writes an (out, max, sum) part
+// and gqa_combine_kernel merges the parts of a row: the same softmax over the same positions either way (f32
+// throughout, probabilities enter the V product as bf16 hi + lo); only the order of the f32 sums differs.
 
 template <int H>
 struct PrefixLds {
@@ -229,32 +234,37 @@ struct PrefixLds {
   float m[2][32], l[2][32];
 };
 
+// What one workgroup of the tile walk does.
+struct TileJob {
+  int kv_row;      // sequence whose cache rows and mask entries are read
+  int row0, nrows; // query rows row0 .. row0 + nrows - 1 (nrows <= 32 / G), all heads of the kv head
+  int pbeg, pend;  // positions [pbeg, pend)
+  int split, nsp;  // this workgroup takes split `split` of nsp splits of the blocks of 32 positions
+  int part;        // index of the part it writes when a row has several (nparts > 1)
+  int nparts;
+};
+
 template <int H, int G>
-__device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>& lds, const int kvh, const int gq,
-                                                const int ps) {
+__device__ __forceinline__ void gqa_tile_walk(const AttnArgs& a, PrefixLds<H>& lds, const int kvh, const TileJob j) {
   constexpr int KS = H / 16;        // MFMA k-steps of the score product
   constexpr int CPR = H / 8;        // 16-byte chunks per cache row
   constexpr int RPD = 64 / CPR;     // rows per 1 KiB direct-to-LDS load
   constexpr int NLD = 32 / RPD;     // loads per wave and V tile
   constexpr int HT = H / 32;        // hidden tiles of the output
-  constexpr int RPB = 32 / G;       // sequences per query block
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int h = lane >> 5, qi = lane & 31;
-  const int qblocks = (a.share_gs + RPB - 1) / RPB;
-  const int grp = gq / qblocks, qb = gq - grp * qblocks;
-  const int lead = grp * a.share_gs;  // the group's first sequence: its cache rows and mask are the ones read
-  const int step = min(*a.step, min(a.C, a.buf_len) - 1);
-  const int plen = min(a.share_len, step + 1);
-  const int nblk = (plen + 31) >> 5;
-  const int bps = (nblk + a.psplits - 1) / a.psplits;
-  const int b_end = min((ps + 1) * bps, nblk);
+  const int lead = j.kv_row;
+  const int plen = j.pend - j.pbeg;  // positions are counted from pbeg below
+  const int nblk = plen > 0 ? (plen + 31) >> 5 : 0;
+  const int bps = (nblk + j.nsp - 1) / j.nsp;
+  const int b_end = min((j.split + 1) * bps, nblk);
 
-  // query fragments of the block into LDS: thread (query, chunk) copies 16 bytes; rows past the group
-  // repeat its last sequence (their results are not stored)
+  // query fragments of the block into LDS: thread (query, chunk) copies 16 bytes; columns past the block's
+  // rows repeat its last row (their results are not stored)
   for (int e = threadIdx.x; e < 32 * CPR; e += 256) {
     const int q = e / CPR, c = e % CPR;
-    const int lr = min(qb * RPB + q / G, a.share_gs - 1);
-    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)(lead + lr) * a.N + kvh * G + q % G) * H + c * 8);
+    const int lr = min(q / G, j.nrows - 1);
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)(j.row0 + lr) * a.N + kvh * G + q % G) * H + c * 8);
     *reinterpret_cast<u32x4_t*>(lds.q + (c * 32 + q) * 8) = v;
   }
   __syncthreads();
@@ -274,7 +284,7 @@ __device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>&
     asm volatile("" : "+v"(sw));
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
-      load_row_to_lds(rv, vt + i * RPD * H, vrow + ((sw ^ ((i * RPD) % CPR)) << 4), (blk * 32 + i * RPD) * row_bytes);
+      load_row_to_lds(rv, vt + i * RPD * H, vrow + ((sw ^ ((i * RPD) % CPR)) << 4), (j.pbeg + blk * 32 + i * RPD) * row_bytes);
   };
   // K fragments of a block: lane (position qi, h) reads the half h of its row, 16 bytes per MFMA step
   const int koff = qi * row_bytes + h * H;
@@ -282,11 +292,11 @@ __device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>&
   auto load_k = [&](int blk) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < KS; ++t)
-      kf[t] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rk, koff + t * 16, blk * 32 * row_bytes, 0));
+      kf[t] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rk, koff + t * 16, (j.pbeg + blk * 32) * row_bytes, 0));
   };
   const uint8_t* mrow = a.input_mask + (size_t)lead * a.buf_len;
   auto mask_byte = [&](int blk) __attribute__((always_inline)) {
-    const int p = blk * 32 + qi;
+    const int p = j.pbeg + blk * 32 + qi;
     return (h == 0 && p < a.buf_len) ? mrow[p] : (uint8_t)0;
   };
 
@@ -297,7 +307,7 @@ __device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>&
     for (int r = 0; r < 16; ++r) o[c][r] = 0.f;
   float m = -1e30f, l = 0.f;
 
-  int blk = ps * bps + wave;
+  int blk = j.split * bps + wave;
   uint8_t mb = 0;
   if (blk < b_end) {
     mb = mask_byte(blk);
@@ -321,7 +331,7 @@ __device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>&
     // accumulator register r holds position 8 (r / 4) + 4 h + r % 4 of the block: with the lane's half folded
     // into the mask word and the limit, the per-register part is a compile-time constant
     const uint32_t mb2 = mbits >> (4 * h);
-    const int lim = plen - blk * 32 - 4 * h;
+    const int lim = plen - blk * 32 - 4 * h;  // plen: positions of this walk, counted from pbeg
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int pc = (r >> 2) * 8 + (r & 3);
@@ -428,11 +438,25 @@ __device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>&
   __syncthreads();
   if (wave != 0) return;
   take(0);
-  // wave 0 holds out^T [hidden, query] for the block's queries: one part per (sequence, query head)
-  const int lr = qb * RPB + qi / G, g = qi % G;
-  if (lr >= a.share_gs) return;
-  const int nparts = a.nsplit + a.psplits;
-  float* pr = a.partial + ((((size_t)(lead + lr) * a.Kh + kvh) * nparts + a.nsplit + ps) * G + g) * (H + 2);
+  // wave 0 holds out^T [hidden, query] for the block's queries
+  const int lr = qi / G, g = qi % G;
+  if (lr >= j.nrows) return;
+  const int row = j.row0 + lr;
+  if (j.nparts == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    uint16_t* dst = a.out + ((size_t)row * a.N + kvh * G + g) * H;
+#pragma unroll
+    for (int c = 0; c < HT; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint2 w;
+        w.x = pack_bf2(o[c][4 * i] * inv, o[c][4 * i + 1] * inv);
+        w.y = pack_bf2(o[c][4 * i + 2] * inv, o[c][4 * i + 3] * inv);
+        *reinterpret_cast<uint2*>(dst + 32 * c + 8 * i + 4 * h) = w;
+      }
+    return;
+  }
+  float* pr = a.partial + ((((size_t)row * a.Kh + kvh) * j.nparts + j.part) * G + g) * (H + 2);
 #pragma unroll
   for (int c = 0; c < HT; ++c)
 #pragma unroll
@@ -449,21 +473,64 @@ __device__ __forceinline__ void gqa_prefix_walk(const AttnArgs& a, PrefixLds<H>&
   }
 }
 
-// One launch for both walks: blockIdx.y below n_prefix_y = (group, query block) of the shared slots, the rest one
-// row each (the groups' workgroups first in dispatch order).  Three workgroups per CU (LDS and registers), so
-// that the rows' workgroups and the groups' are all resident at a rollout's batch sizes.
+// The job of workgroup (y, z) of a launch whose first n_group_y y-indices are (group, query block) pairs of the
+// shared slots and whose other y-indices are rows; false: nothing to do.
+template <int G>
+__device__ __forceinline__ bool tile_job(const AttnArgs& a, int n_group_y, int y, int z, bool rows_too, TileJob& j) {
+  constexpr int RPB = 32 / G;  // sequences per query block
+  // newest valid slot; clamped into the cache and the mask row so that a caller that oversteps reads in bounds
+  const int step = min(*a.step, min(a.C, a.buf_len) - 1);
+  const int shared_end = a.share_gs > 1 ? min(a.share_len, step + 1) : 0;
+  j.nparts = a.nsplit + a.psplits;
+  j.split = z;
+  if (y < n_group_y) {
+    if (z >= a.psplits) return false;
+    const int qblocks = (a.share_gs + RPB - 1) / RPB;
+    const int grp = y / qblocks, qb = y - grp * qblocks;
+    j.kv_row = grp * a.share_gs;
+    j.row0 = j.kv_row + qb * RPB;
+    j.nrows = min(RPB, a.share_gs - qb * RPB);
+    j.pbeg = 0; j.pend = shared_end;
+    j.nsp = a.psplits;
+    j.part = a.nsplit + z;
+    return true;
+  }
+  if (!rows_too || z >= a.nsplit) return false;
+  j.kv_row = j.row0 = y - n_group_y;
+  j.nrows = 1;
+  j.pbeg = shared_end; j.pend = step + 1;
+  j.nsp = a.nsplit;
+  j.part = z;
+  return true;
+}
+
+// grid (Kh, group query blocks + rows, splits): every workgroup runs the tile walk (the groups' workgroups first
+// in dispatch order).  Three workgroups per CU (LDS and registers).
 template <int H, int G>
-__global__ __launch_bounds__(256, 3) void gqa_shared_kernel(AttnArgs a, int n_prefix_y) {
+__global__ __launch_bounds__(256, 3) void gqa_tile_kernel(AttnArgs a, int n_group_y) {
+  __shared__ PrefixLds<H> lds;
+  TileJob j;
+  if (tile_job<G>(a, n_group_y, blockIdx.y, blockIdx.z, true, j)) gqa_tile_walk<H, G>(a, lds, blockIdx.x, j);
+}
+
+// The same grid with the rows' own slots on the vector-ALU walk (gqa_decode_walk) and only the shared slots on
+// the tile walk: up to four query heads per kv head the vector walk streams cold cache rows faster (whole rows
+// in coalesced non-temporal loads; the tile walk fetches K in 16-byte pieces per lane): measured on the 8B
+// rollout shape, 64 sequences at context 512, per decode step: 3.997 ms this way, 4.098 ms all on the tile
+// walk, 4.176 ms without sharing.
+template <int H, int G>
+__global__ __launch_bounds__(256, 3) void gqa_shared_kernel(AttnArgs a, int n_group_y) {
   union Lds {
     DecodeLds<H, G> d;
     PrefixLds<H> p;
   };
   __shared__ Lds lds;
-  if ((int)blockIdx.y < n_prefix_y) {
-    if ((int)blockIdx.z < a.psplits) gqa_prefix_walk<H, G>(a, lds.p, blockIdx.x, blockIdx.y, blockIdx.z);
+  if ((int)blockIdx.y < n_group_y) {
+    TileJob j;
+    if (tile_job<G>(a, n_group_y, blockIdx.y, blockIdx.z, false, j)) gqa_tile_walk<H, G>(a, lds.p, blockIdx.x, j);
     return;
   }
-  if ((int)blockIdx.z < a.nsplit) gqa_decode_walk<H, G>(a, lds.d, blockIdx.x, (int)blockIdx.y - n_prefix_y, blockIdx.z);
+  if ((int)blockIdx.z < a.nsplit) gqa_decode_walk<H, G>(a, lds.d, blockIdx.x, (int)blockIdx.y - n_group_y, blockIdx.z);
 }
 
 // ---------------------------------------------------------------------------
@@ -649,8 +716,8 @@ static int launch_attn(hipStream_t st, const AttnArgs& a) {
   return check_launch();
 }
 
-// Number of sequence splits that brings the grid to roughly two workgroups per CU (more splits
-// cost more in partial sums and the combine launch than they gain at rollout batch sizes).
+// Number of sequence splits of the vector-ALU walk that brings the grid to roughly two workgroups per CU
+// (more splits cost more in partial sums and the combine launch than they gain at rollout batch sizes).
 // Mid-sized grids (65 to 256 (sequence, kv head) pairs, the 30B-A3B shape at 32 sequences) run
 // fastest at four workgroups per CU with chunks down to 128 positions (measured).
 int attn_num_splits(int B, int Kh, int C) {
@@ -665,65 +732,118 @@ int attn_num_splits(int B, int Kh, int C) {
   return ns;
 }
 
-size_t attn_partial_bytes(int B, int N, int Kh, int H, int C) {
-  const int ns = attn_num_splits(B, Kh, C);
-  return ns == 1 ? 0 : (size_t)B * N * ns * (H + 2) * sizeof(float);
-}
-
-// Splits of the shared slots: two waves of a workgroup get one block of 32 positions each, up to
-// kMaxPrefixSplits workgroups per (group, kv head, query block) (measured on 256 shared slots at 64 sequences:
-// 1, 2, 4 splits -> 23.9, 22.1, 21.2 us for the launch; the combine launch behind it reads one more part per split).
-static int prefix_splits(int share_len) {
-  const int nblk = (share_len + 31) / 32;
-  int ps = nblk / 2;
-  if (ps < 1) ps = 1;
-  return ps > kMaxPrefixSplits ? kMaxPrefixSplits : ps;
-}
-
-size_t attn_shared_partial_bytes(int B, int N, int Kh, int H, int C) {
-  return (size_t)B * N * (attn_num_splits(B, Kh, C) + kMaxPrefixSplits) * (H + 2) * sizeof(float);
-}
-
-// The shared walk serves one token per sequence, up to 128 sequences in whole groups, head dimensions and
-// group widths of the MFMA tile (G query heads per kv head, G in {1, 2, 4}), and 32-bit byte offsets per cache.
+// The shared walk serves one token per sequence, up to 128 sequences in whole groups, the head dimensions and
+// group widths of the tile walk, and 32-bit byte offsets per cache.
 bool attn_share_ok(int B, int N, int Kh, int H, int C, int share_gs, int share_len) {
   if (share_gs <= 1 || share_len < 32 || share_len > C || B <= 0 || B > 128 || B % share_gs) return false;
   if (Kh <= 0 || N % Kh || (H != 64 && H != 128)) return false;
   const int G = N / Kh;
-  if (G != 1 && G != 2 && G != 4) return false;
+  if (G != 1 && G != 2 && G != 4 && G != 8) return false;
   return (size_t)C * Kh * H * 2 < (1u << 31);
 }
 
+// Which kernel walks the cache of a one-token step, and in how many splits.
+struct AttnPlan {
+  bool tile;    // gqa_tile_kernel (matrix pipe) or gqa_decode_kernel (vector ALU)
+  bool shared;  // tile only: prompt slots once per group
+  int nsplit;   // splits of a row's own slots
+  int psplits;  // splits of the shared slots
+};
+
+static AttnPlan plan_attention(int B, int N, int Kh, int H, int C, int share_gs, int share_len) {
+  AttnPlan p = {false, false, attn_num_splits(B, Kh, C), 0};
+  const int G = Kh > 0 && N % Kh == 0 ? N / Kh : 0;
+  if ((H != 64 && H != 128) || (G != 1 && G != 2 && G != 4 && G != 8) || (size_t)C * Kh * H * 2 >= (1u << 31)) return p;
+  // Launches with tile-walk workgroups hold three per CU and want them all resident at once (measured at 128
+  // sequences x 8 kv heads = 1024 workgroups: 108 against 98 us for the vector-ALU walk, four of whose workgroups
+  // fit a CU); with shared prompt slots a launch reads fewer cache rows and may take two rounds.
+  const long slots = 3L * device_cus(), pairs = (long)B * Kh;
+  p.shared = attn_share_ok(B, N, Kh, H, C, share_gs, share_len);
+  // Rows' own slots: the tile walk for 8 query heads per kv head (measured on the 30B-A3B shape, 32 sequences at
+  // context 512: 10.7 + 3.0 us for walk and combine against 21.7 + 3.9 us; the vector walk's work per cache row
+  // grows with the heads); up to 4 heads the vector walk (see gqa_shared_kernel).
+  p.tile = G == 8 && pairs <= (p.shared ? 2 * slots : slots);
+  if (G == 8 && !p.tile) p.shared = false;
+  if (p.shared && pairs > 2 * slots) p.shared = false;
+  long group_wgs = 0;
+  if (p.shared) {
+    const int rpb = 32 / G, qblocks = (share_gs + rpb - 1) / rpb;
+    group_wgs = (long)(B / share_gs) * qblocks * Kh;
+    // splits of the shared slots: a block of 32 positions for every other wave, while the launch stays resident
+    // (measured on 256 shared slots at 64 sequences of the 8B shape: 1, 2, 4 splits -> 23.9, 22.1, 21.2 us)
+    const int nblk = (share_len + 31) / 32;
+    p.psplits = nblk / 2 < 1 ? 1 : (nblk / 2 > kMaxPrefixSplits ? kMaxPrefixSplits : nblk / 2);
+    while (p.psplits > 1 && pairs + group_wgs * p.psplits > slots) --p.psplits;
+  }
+  if (p.tile) {
+    // fill the slots that are left, at least 8 blocks of 32 positions per split
+    long ns = (slots - group_wgs * p.psplits) / pairs;
+    const int by_len = (C + 255) / 256;
+    if (ns > by_len) ns = by_len;
+    if (ns > 8) ns = 8;
+    p.nsplit = ns < 1 ? 1 : (int)ns;
+  } else if (p.shared) {
+    p.nsplit = 1;  // the vector walk behind shared slots: one split per row (more did not pay, see above)
+  }
+  return p;
+}
+
+size_t attn_partial_bytes(int B, int N, int Kh, int H, int C) {
+  const AttnPlan p = plan_attention(B, N, Kh, H, C, 0, 0);
+  // rows of two or three tokens per pass take the vector-ALU walk whatever the plan says
+  const int ns = p.nsplit > attn_num_splits(B, Kh, C) ? p.nsplit : attn_num_splits(B, Kh, C);
+  return ns == 1 ? 0 : (size_t)B * N * ns * (H + 2) * sizeof(float);
+}
+
+// room for every plan of this shape, shared slots included
+size_t attn_shared_partial_bytes(int B, int N, int Kh, int H, int C) {
+  const int nv = attn_num_splits(B, Kh, C);
+  const int ns = nv > 8 ? nv : 8;
+  return (size_t)B * N * (ns + kMaxPrefixSplits) * (H + 2) * sizeof(float);
+}
+
 template <int H, int G>
-static int launch_shared(hipStream_t st, const AttnArgs& a) {
-  const int rpb = 32 / G, qblocks = (a.share_gs + rpb - 1) / rpb;
-  const int n_prefix_y = (a.B / a.share_gs) * qblocks;
+static int launch_tile(hipStream_t st, const AttnArgs& a, bool rows_on_tile) {
+  int n_group_y = 0;
+  if (a.share_gs > 1) {
+    const int rpb = 32 / G, qblocks = (a.share_gs + rpb - 1) / rpb;
+    n_group_y = (a.B / a.share_gs) * qblocks;
+  }
   const int nz = a.nsplit > a.psplits ? a.nsplit : a.psplits;
-  hipLaunchKernelGGL((gqa_shared_kernel<H, G>), dim3(a.Kh, n_prefix_y + a.B, nz), dim3(256), 0, st, a, n_prefix_y);
+  const dim3 grid(a.Kh, n_group_y + a.B, nz);
+  if (rows_on_tile) hipLaunchKernelGGL((gqa_tile_kernel<H, G>), grid, dim3(256), 0, st, a, n_group_y);
+  else if constexpr (G <= 4) hipLaunchKernelGGL((gqa_shared_kernel<H, G>), grid, dim3(256), 0, st, a, n_group_y);
+  else return TMX_ERR_UNSUPPORTED;
   int rc = check_launch();
-  if (rc != TMX_OK) return rc;
+  if (rc != TMX_OK || a.nsplit + a.psplits == 1) return rc;
   hipLaunchKernelGGL((gqa_combine_kernel<H, G>), dim3(a.Kh, a.B, G), dim3(H), 0, st, a);
   return check_launch();
 }
 
 int gqa_decode(hipStream_t st, AttnArgs a, int H) {
-  a.nsplit = attn_num_splits(a.B, a.Kh, a.C);
   const int G = a.N / a.Kh;
   if (a.N % a.Kh) return TMX_ERR_SHAPE;
-  if (a.tpp <= 1 && attn_share_ok(a.B, a.N, a.Kh, H, a.C, a.share_gs, a.share_len)) {
-    // G samples of a prompt in consecutive rows: the prompt slots once per group, the rest per row
-    if (!a.partial) return TMX_ERR_ARG;
-    a.psplits = prefix_splits(a.share_len);
-#define TMX_SHARED_CASE(HH, GG) \
-  if (H == HH && G == GG) return launch_shared<HH, GG>(st, a);
-    TMX_SHARED_CASE(64, 1)
-    TMX_SHARED_CASE(64, 2)
-    TMX_SHARED_CASE(64, 4)
-    TMX_SHARED_CASE(128, 1)
-    TMX_SHARED_CASE(128, 2)
-    TMX_SHARED_CASE(128, 4)
-#undef TMX_SHARED_CASE
+  if (a.tpp <= 1) {
+    const AttnPlan p = plan_attention(a.B, a.N, a.Kh, H, a.C, a.share_gs, a.share_len);
+    if (p.tile || p.shared) {
+      a.nsplit = p.nsplit;
+      a.psplits = p.shared ? p.psplits : 0;
+      if (!p.shared) a.share_gs = a.share_len = 0;
+      if (a.nsplit + a.psplits > 1 && !a.partial) return TMX_ERR_ARG;
+#define TMX_TILE_CASE(HH, GG) \
+  if (H == HH && G == GG) return launch_tile<HH, GG>(st, a, p.tile);
+      TMX_TILE_CASE(64, 1)
+      TMX_TILE_CASE(64, 2)
+      TMX_TILE_CASE(64, 4)
+      TMX_TILE_CASE(64, 8)
+      TMX_TILE_CASE(128, 1)
+      TMX_TILE_CASE(128, 2)
+      TMX_TILE_CASE(128, 4)
+      TMX_TILE_CASE(128, 8)
+#undef TMX_TILE_CASE
+    }
   }
+  a.nsplit = attn_num_splits(a.B, a.Kh, a.C);
   a.share_gs = a.share_len = a.psplits = 0;
   if (a.nsplit > 1 && !a.partial) return TMX_ERR_ARG;
   // several tokens per sequence: one walk over the cache for a block of them (MFMA kernel)
@@ -790,7 +910,7 @@ extern "C" int tmx_gqa_decode_attention_shared(void* stream, const void* q, cons
                                                int share_group, int share_len) {
   if (!q || !kcache || !vcache || !input_mask || !step || !out || !workspace) return TMX_ERR_ARG;
   if (B <= 0 || N <= 0 || Kh <= 0 || C <= 0) return TMX_ERR_SHAPE;
-  if (!attn_share_ok(B, N, Kh, H, C, share_group, share_len)) return TMX_ERR_UNSUPPORTED;
+  if (!plan_attention(B, N, Kh, H, C, share_group, share_len).shared) return TMX_ERR_UNSUPPORTED;
   AttnArgs a = {};
   a.q = (const uint16_t*)q;
   a.kcache = (const uint16_t*)kcache;
