@@ -254,33 +254,46 @@ def main():
     dst.copy_(src)  # reads 1 GiB, writes 1 GiB
     torch.cuda.synchronize()
     del src, dst
-  st = fresh_state()
-  run(st, args.warmup)
-  torch.cuda.synchronize()
-  t0 = time.perf_counter()
-  run(st, args.steps)
-  torch.cuda.synchronize()
-  dt = time.perf_counter() - t0
-  toks = st['token_buffer'][:, start:start + args.warmup + args.steps]
-  assert int(st['step'].item()) == start - 1 + args.warmup + args.steps
-  assert bool(((toks >= 0) & (toks < cfg.vocab_size)).all().item())
-  lps = st['logprobs'][:, start:start + args.warmup + args.steps]
-  assert bool(torch.isfinite(lps).all().item()) and bool((lps <= 0).all().item())
-  # a hand-over inside a launch whose bounded wait ran out would have dropped a LoRA term: raises if so
-  sampler.check_device_status(st)
+  def timed_run():
+    st = fresh_state()
+    run(st, args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run(st, args.steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    toks = st['token_buffer'][:, start:start + args.warmup + args.steps]
+    assert int(st['step'].item()) == start - 1 + args.warmup + args.steps
+    assert bool(((toks >= 0) & (toks < cfg.vocab_size)).all().item())
+    lps = st['logprobs'][:, start:start + args.warmup + args.steps]
+    assert bool(torch.isfinite(lps).all().item()) and bool((lps <= 0).all().item())
+    # a hand-over inside a launch whose bounded wait ran out would have dropped a LoRA term: raises if so
+    sampler.check_device_status(st)
+    return st, dt
+
+  # The product's own path first: where consecutive rows hold samples of one prompt (the GRPO workload), decode
+  # attention reads the prompt slots once per group.  Every roofline figure below prices the K/V bytes at
+  # sequences x context and therefore comes from a second run WITHOUT that sharing (the same launches otherwise).
+  st, dt = timed_run()
+  shared = (st['share_group'], st['share_len']) if st['share_group'] > 1 else None
+  dt_product, walk_product = dt, walk_ms[0]
+  if shared:
+    sampler.share_prompt_kv = False
+    walk_ms.clear()
+    st, dt = timed_run()
 
   result = {
       'metric': f'generated tokens/s at 1 GPU, int4 QLoRA {LABELS[args.workload]} rollout (decode)',
-      'value': batch * args.steps / dt,
+      'value': batch * args.steps / dt_product,
       'unit': 'tokens/s',
       'n_gpus': 1,
       'steps': args.steps,
       'warmup': args.warmup,
-      'ms_per_step': dt / args.steps * 1e3,
+      'ms_per_step': dt_product / args.steps * 1e3,
       'higher_is_better': True,
       'scaling': 'weak',
       'vs_baseline': None,
-      'cache_fill_ms': walk_ms[0],
+      'cache_fill_ms': walk_product,
       'dtype': 'bf16 activations / int4 weights / f32 accumulate',
       'data': 'synthetic (random-init weights, uniform-random prompt ids)',
       'config': {
@@ -300,6 +313,18 @@ def main():
   result['step_hbm'] = {'algorithmic_bytes': step_bytes,
                         'achieved_GBps': step_bytes / (dt / args.steps) / 1e9,
                         'frac_of_8TBps': step_bytes / (dt / args.steps) / 8e12}
+  if shared:
+    # beside, not inside, the figures priced at sequences x context: step_hbm, roofline and kernel_ms_per_step are
+    # the run without sharing; `value` / `ms_per_step` are the product's default path (sharing on)
+    result['prompt_kv_sharing'] = {
+        'share_group': shared[0], 'share_len': shared[1],
+        'value': batch * args.steps / dt_product, 'ms_per_step': dt_product / args.steps * 1e3,
+        'value_without': batch * args.steps / dt, 'ms_per_step_without': dt / args.steps * 1e3,
+        'kv_rows_read_per_step_ratio': (batch * (s_mean - shared[1]) + batch / shared[0] * shared[1]) / (batch * s_mean),
+        'cache_fill_ms': walk_product, 'cache_fill_ms_without': walk_ms[0],
+        'note': 'step_hbm, roofline* and kernel_ms_per_step below are measured WITHOUT sharing (K/V bytes priced at '
+                'sequences x context); value and ms_per_step are the default path, which reads the prompt slots '
+                'once per group of samples of one prompt'}
 
   if not args.no_profile:
     # Replay the same rollout with HIP events around every launch: every 8th step of a long run,
@@ -494,6 +519,25 @@ def main():
     }
     del xs, yp, tp
 
+  if shared and not args.no_profile:
+    # the attention launch of the default path, timed the same way over a few steps
+    sampler.share_prompt_kv = True
+    lib = _lib.lib()
+    st = fresh_state()
+    sampler.run_steps(st, args.warmup, sample=True)
+    ms = np.zeros(len(CLASS_NAMES), np.float32)
+    cnt = np.zeros(len(CLASS_NAMES), np.int32)
+    tot = 0.0
+    n_prof = min(8, args.steps)
+    for _ in range(n_prof):
+      cs = sampler._c_state(st)
+      rc = lib.tmx_decode_steps_profiled(ctypes.byref(model.desc()), ctypes.byref(cs), _lib.stream(), 1, 1,
+                                         ms.ctypes.data_as(ctypes.c_void_p), cnt.ctypes.data_as(ctypes.c_void_p))
+      _lib.check(rc, 'tmx_decode_steps_profiled')
+      tot += float(ms[CLASS_NAMES.index('attention')])
+    sampler.check_device_status(st)
+    result['prompt_kv_sharing']['attention_ms_per_step'] = tot / n_prof
+    result['prompt_kv_sharing']['attention_ms_per_step_without'] = result['kernel_ms_per_step']['attention']
   if not args.no_cpu_baseline and not cfg.num_experts:
     del st
     result['cpu_baseline'] = cpu_baseline(args.workload)

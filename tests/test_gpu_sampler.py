@@ -219,7 +219,7 @@ def test_samples_of_one_prompt_share_its_cache_rows_and_match_oracle():
     s.eos_ids = np.array([-1])
     st = s.init_sample_state(ids, p + 10, True, None, 0.0, None, None, 0, include_logprobs=True,
                              prompt_lengths=ref['prompt_lengths'])
-    assert (st['share_group'], st['share_len']) == ((4, p // 32 * 32) if share else (1, 0))
+    assert (st['share_group'], st['share_len'], st['share_common']) == ((4, p // 32 * 32, p) if share else (1, 0, 0))
     s.walk(st, p - 1)
     steps = []
     for step in range(10):

@@ -350,3 +350,26 @@ def test_host_code_under_address_and_undefined_sanitizers():
   assert res.returncode == 0, res.stdout + res.stderr
   assert 'host sanitizer run ok' in res.stdout
   assert 'AddressSanitizer' not in res.stderr and 'runtime error' not in res.stderr, res.stderr
+
+
+def test_shared_prompt_groups_are_found_on_the_host():
+  """Rows that hold samples of one prompt (tunix/rl/rl_learner.py:432-435: every prompt repeated
+  num_generations times, consecutively) are grouped by the columns they have in common; a differing mask or
+  token ends the common part, and a batch of distinct prompts shares nothing."""
+  from tunix_amd.sampler import shared_prompt_groups as groups
+  rng = np.random.default_rng(0)
+  base = rng.integers(3, 100, (8, 256))
+  ids = np.repeat(base, 8, axis=0)
+  ones = lambda a: np.ones_like(a, bool)
+  assert groups(ids, ones(ids)) == (8, 256, 256)
+  tail = np.concatenate([ids, rng.integers(3, 100, (64, 200))], axis=1)   # private columns behind the prompt
+  assert groups(tail, ones(tail)) == (8, 256, 256)
+  assert groups(base, ones(base)) == (1, 0, 0)
+  odd = np.repeat(rng.integers(3, 100, (2, 70)), 4, axis=0)
+  assert groups(odd, ones(odd)) == (4, 64, 70)                             # 70 common columns, 64 = two blocks of 32
+  odd[5, 40] = 1
+  assert groups(odd, ones(odd)) == (4, 32, 40)
+  m = ones(ids)
+  m[3, 10] = False                                                          # one row masks a column: not the same prompt any more
+  assert groups(ids, m)[1] < 32 or groups(ids, m)[0] != 8
+  assert groups(ids[:, :16], ones(ids[:, :16])) == (1, 0, 0)               # too short to be worth a launch of its own

@@ -77,25 +77,27 @@ def _seed_key(seed):
 
 
 def shared_prompt_groups(ids, mask, min_len=32, max_group=64):
-  """(g, n): the largest saving split of the rows into consecutive groups of g whose first n columns agree
-  in token ids and mask; (1, 0) when nothing is worth sharing.  A GRPO rollout decodes the G samples of a
-  prompt as consecutive rows (tunix/rl/rl_learner.py:432-435 repeats every prompt num_generations times), so
-  the K / V rows of the prompt columns are the same within a group and decode attention can read them once
-  per group.  n is rounded down to a multiple of 32; the saving counted is (g - 1) / g * n cache rows."""
+  """(g, n, c): the largest saving split of the rows into consecutive groups of g whose first c columns agree
+  in token ids and mask, n = c rounded down to a multiple of 32; (1, 0, 0) when nothing is worth sharing.  A
+  GRPO rollout decodes the G samples of a prompt as consecutive rows (tunix/rl/rl_learner.py:432-435 repeats
+  every prompt num_generations times), so the K / V rows of the prompt columns are the same within a group:
+  decode attention reads n of them once per group, and the cache fill computes c of them once per group.  The
+  saving counted is (g - 1) / g * n cache rows."""
   ids, mask = np.asarray(ids), np.asarray(mask)
   b, p = ids.shape
   if b < 2 or p < min_len:
-    return 1, 0
+    return 1, 0, 0
   same = (ids[1:] == ids[:-1]) & (mask[1:] == mask[:-1])          # row i + 1 against row i, per column
   run = np.where(same.all(axis=1), p, np.argmin(same, axis=1))   # columns in which row i + 1 repeats row i
-  best, best_gain = (1, 0), 0.0
+  best, best_gain = (1, 0, 0), 0.0
   for g in range(2, min(b, max_group) + 1):
     if b % g:
       continue
     inner = np.arange(1, b) % g != 0                              # pairs (i, i + 1) inside one group
-    n = int(run[inner[: b - 1]].min()) // 32 * 32
+    c = int(run[inner[: b - 1]].min())
+    n = c // 32 * 32
     if n >= min_len and (g - 1) / g * n > best_gain:
-      best, best_gain = (g, n), (g - 1) / g * n
+      best, best_gain = (g, n, c), (g - 1) / g * n
   return best
 
 
@@ -170,6 +172,7 @@ class Sampler:
 
   def delete_cache(self):
     self._cache = None
+    self._lead_cache = None
     self._workspace = None
 
   def reinitialize_cache(self):
@@ -204,7 +207,7 @@ class Sampler:
     else:
       input_mask[:, :p] = ids != pad
     positions = utils.build_positions_from_mask(input_mask)
-    share = shared_prompt_groups(ids, input_mask[:, :p]) if self.share_prompt_kv else (1, 0)
+    share = shared_prompt_groups(ids, input_mask[:, :p]) if self.share_prompt_kv else (1, 0, 0)
     c = self._transformer.config
     need = (c.num_layers, 2, b, self.cache_config.cache_size, c.num_kv_heads, c.head_dim)
     if self._cache is None or tuple(self._cache.shape) != need:
@@ -224,7 +227,8 @@ class Sampler:
         'step': torch.zeros(1, dtype=torch.int32, device=dev),
         'cache': self._cache,
         'num_input_tokens': p,
-        'share_group': share[0], 'share_len': share[1],
+        'share_group': share[0], 'share_len': share[1], 'share_common': share[2],
+        'fresh': True,  # nothing walked yet: the cache fill may start with one pass per group of equal prompts
         'total_sampling_steps': total_sampling_steps,
         'sampling_mode': 'greedy' if top_p is None else 'top_p',
         'temperature': float(temperature),
@@ -306,6 +310,12 @@ class Sampler:
     MAX_ROWS rows (MAX_FILL_ROWS without the head, where the model allows), instead of one
     token per launch sequence."""
     b = st['token_buffer'].shape[0]
+    if st.get('fresh') and not sample and st.get('share_group', 1) > 1:
+      n_lead = min(n_tokens, st['share_common'])
+      if n_lead >= 32:
+        self._walk_group_leaders(st, n_lead)
+        n_tokens -= n_lead
+    st['fresh'] = False
     # the head chooses tokens for up to MAX_ROWS rows; scoring takes as many rows as a cache fill
     choose = sample and st['sampling_mode'] != 'score'
     per = min(128, max(1, (self.MAX_ROWS if choose else self._fill_rows()) // b))
@@ -320,6 +330,31 @@ class Sampler:
         # thousands of short passes otherwise leaves tens of thousands of dispatches pending at once
         torch.cuda.current_stream().synchronize()
 
+  def _walk_group_leaders(self, st, n):
+    """Cache fill over the first n columns, which every group of st['share_group'] consecutive rows has in
+    common (the samples of one prompt): the first row of every group is walked, in a cache of its own, and
+    its K / V rows are copied to the cache rows of the whole group, so the prompt is computed once per group
+    instead of once per sample.  Advances st['step'] by n like a walk over all rows."""
+    g = st['share_group']
+    b = st['token_buffer'].shape[0]
+    dev = self._transformer.device
+    lead = torch.arange(0, b, g, device=dev)
+    c = self._transformer.config
+    need = (c.num_layers, 2, b // g, self.cache_config.cache_size, c.num_kv_heads, c.head_dim)
+    if getattr(self, '_lead_cache', None) is None or tuple(self._lead_cache.shape) != need:
+      self._lead_cache = None
+      self._lead_cache = self._transformer.init_cache(b // g, self.cache_config.cache_size)
+    sub = dict(st)
+    sub.update({
+        'token_buffer': st['token_buffer'][lead].contiguous(), 'positions': st['positions'][lead].contiguous(),
+        'input_mask': st['input_mask'][lead].contiguous(), 'done': torch.zeros(b // g, dtype=torch.uint8, device=dev),
+        'logprobs': None, 'logits': None, 'step': torch.zeros(1, dtype=torch.int32, device=dev),
+        'cache': self._lead_cache, 'share_group': 1, 'share_len': 0, 'share_common': 0, 'fresh': False})
+    self.walk(sub, n)
+    for r in range(g):  # rows r, r + g, ... of the cache <- the leaders' rows (strided copies, no temporary)
+      st['cache'][:, :, r::g, :n].copy_(self._lead_cache[:, :, :, :n])
+    st['step'].fill_(n)
+
   def run_steps(self, st, n_steps, sample=True, graph=False, tokens_per_pass=1):
     """Runs n decode-loop iterations on the current stream.  graph=False only enqueues (no host
     sync); graph=True replays one recorded step and returns when the steps have run.
@@ -327,6 +362,7 @@ class Sampler:
     (cache fill or scoring only)."""
     if n_steps <= 0:
       return
+    st['fresh'] = False
     cs = self._c_state(st, tokens_per_pass)
     fn = self._lib.tmx_decode_steps_graph if graph else self._lib.tmx_decode_steps
     rc = fn(ctypes.byref(self._transformer.desc()), ctypes.byref(cs), _lib.stream(), int(n_steps),
