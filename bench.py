@@ -420,7 +420,7 @@ def main():
     for cls_name, key in dense:
       sym = f'tmx::qlinear_mfma4_kernel<{mt}>' if four(layer0[key]) else kway_symbol(layer0[key])
       symbols.setdefault(sym, []).append(cls_name)
-    small = batch <= 4 and not cfg.num_experts and cfg.family == 'llama3' and tot_cnt[CLASS_NAMES.index('rope_kvwrite')] == 0
+    small = batch <= 4 and not cfg.num_experts and tot_cnt[CLASS_NAMES.index('rope_kvwrite')] == 0
     if small:
       # 1..4 rows: five launches per layer, norm / LoRA / residual / SwiGLU inside the projections
       # (template arguments: prologue 0 plain, 1 norm, 2 attention merge; epilogue 0 plain, 1 residual, 2 SwiGLU)

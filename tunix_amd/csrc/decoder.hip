@@ -41,17 +41,17 @@ static const int kFusedGateUpMaxRows = 64;
 
 struct Splits { int qkv, o, gate_up, down; };
 
-// One to four sequences, one token each, dense Llama-family layers whose shapes fit the small-batch
+// One to four sequences, one token each, dense layers of either family whose shapes fit the small-batch
 // kernels: five launches per layer (see smallbatch.hip).
 static const int kSmallBatchMaxRows = 4;
 static bool small_batch_ok(const tmx_model_desc* m, int B, int T) {
-  if (B > kSmallBatchMaxRows || T != 1 || m->num_experts > 0 || m->family != TMX_FAMILY_LLAMA3) return false;
+  if (B > kSmallBatchMaxRows || T != 1 || m->num_experts > 0) return false;
   const int D = m->embed_dim, N = m->num_heads, Kh = m->num_kv_heads, H = m->head_dim, F = m->hidden_dim;
   const int NH = N * H, QKV = (N + 2 * Kh) * H;
   if (!sb_attn_ok(N, Kh, H)) return false;
   for (int i = 0; i < m->num_layers; ++i) {
     const tmx_layer_desc& l = m->layers[i];
-    if (l.q_norm_w || l.k_norm_w) return false;
+    if ((l.q_norm_w != nullptr) != (l.k_norm_w != nullptr)) return false;
     if (!sb_linear_ok(B, D, QKV, l.qkv.G, l.qkv.lora_a_t ? l.qkv.rank : 0, l.qkv.lora_a_t ? l.qkv.r_pad : 0, true)) return false;
     if (!sb_linear_ok(B, NH, D, l.o.G, l.o.lora_a_t ? l.o.rank : 0, l.o.lora_a_t ? l.o.r_pad : 0, false)) return false;
     if (F % 32 || !sb_linear_ok(B, D, 2 * F, l.gate_up.G, l.gate_up.lora_a_t ? l.gate_up.rank : 0,
@@ -311,6 +311,8 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
           a.partial = w.sb_attn_partial;
           a.B = B; a.N = N; a.Kh = Kh; a.C = C; a.nsplit = ans;
           a.scale = 1.0f / sqrtf((float)H);
+          a.q_norm_w = (const uint16_t*)l.q_norm_w; a.k_norm_w = (const uint16_t*)l.k_norm_w;
+          a.eps = m->norm_eps; a.family = m->family;
           TMX_TRY(TMX_K_ATTN, sb_attn(st, a, H));
         }
         {
@@ -417,18 +419,17 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
         a.residual = w.x; a.x_out = w.x;
         a.norm_w = (const uint16_t*)l.norm2_w; a.xn_out = w.xn;
         a.D = D; a.eps = m->norm_eps; a.family = m->family;
+        if (moe) {
+          // the row's workgroup routes its token from the normed row it has just made: scores, softmax, top-k
+          // (19 us per layer as a launch of its own on the 30B-A3B shape at 32 sequences)
+          a.router.w = (const uint16_t*)l.router_w;
+          a.router.D = D; a.router.E = m->num_experts; a.router.top_k = m->experts_per_tok;
+          a.router.expert_of = w.expert_of; a.router.weight_of = w.weight_of;
+        }
         TMX_TRY(TMX_K_ROWNORM, row_norm(st, a, B));
       }
       if (moe) {
         const int P = B * m->experts_per_tok;
-        {
-          RouterArgs a = {};
-          a.x = w.xn;
-          a.w = (const uint16_t*)l.router_w;
-          a.D = D; a.E = m->num_experts; a.top_k = m->experts_per_tok;
-          a.expert_of = w.expert_of; a.weight_of = w.weight_of;
-          TMX_TRY(TMX_K_ROUTER, moe_route(st, a, B));
-        }
         MoeArgs e = {};
         e.expert_of = w.expert_of; e.P = P; e.top_k = m->experts_per_tok;
         e.x = w.xn; e.ldx = D;

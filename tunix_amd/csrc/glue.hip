@@ -13,7 +13,7 @@
 //   KV write               llama3/model.py:367-377, qwen3/model.py:586-597 (slot = end_index)
 //   residual wiring        llama3/model.py:546-564, qwen3/model.py:1268-1289
 //   SwiGLU                 llama3/model.py:489-496, qwen3/model.py:1199-1208
-#include "tmx_kernels.h"
+#include "tmx_router.h"
 
 namespace tmx {
 
@@ -169,6 +169,7 @@ __device__ __forceinline__ void add_lora8(float* o, const float* t_s, const uint
 // In embedding mode it also fills this step's RoPE sin/cos table row.
 template <int CPT>  // 8-element chunks per thread, D <= 4096 * CPT
 __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
+  extern __shared__ float route_sm[];  // moe_router_lds_floats(D, E) floats when the row is routed here, else none
   __shared__ float smem[8];
   __shared__ float t_s[TMX_MAX_RPAD];
   __shared__ float t_stage[TMX_MAX_LORA_SPLITS * 64];
@@ -327,7 +328,17 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
         else o[e] = w[e] * (v[i][e] / rms);
       }
       *reinterpret_cast<uint4*>(a.xn_out + (size_t)m * a.D + n0) = pack8(o);
+      if (a.router.w) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) route_sm[n0 + e] = rbf(o[e]);
+      }
     }
+  }
+  if (a.router.w) {
+    // MoE layer: the token is routed here, from the normed row this workgroup just made (no router launch, no
+    // reload of xn)
+    __syncthreads();
+    moe_route_token(a.router, route_sm, m);
   }
 }
 
@@ -335,10 +346,18 @@ int row_norm(hipStream_t st, const RowNormArgs& a, int M) {
   if (a.D <= 0 || a.D % 8 || a.D > 4096 * 4) return TMX_ERR_SHAPE;
   if (a.lora.t_part && a.lora.r > TMX_MAX_RPAD) return TMX_ERR_SHAPE;
   if (a.rope_tab && a.half > 256) return TMX_ERR_SHAPE;
+  size_t lds = 0;
+  if (a.router.w) {
+    const RouterArgs& r = a.router;
+    if (!a.norm_w || !r.expert_of || !r.weight_of || r.D != a.D) return TMX_ERR_ARG;
+    if (r.E <= 0 || r.E % 8 || r.top_k <= 0 || r.top_k > 64 || r.top_k > r.E) return TMX_ERR_SHAPE;
+    lds = moe_router_lds_floats(a.D, r.E) * sizeof(float);
+    if (lds > 60000) return TMX_ERR_SHAPE;
+  }
   const int cpt = (a.D / 8 + 511) / 512;
-  if (cpt <= 1) hipLaunchKernelGGL(row_norm_kernel<1>, dim3(M), dim3(512), 0, st, a);
-  else if (cpt <= 2) hipLaunchKernelGGL(row_norm_kernel<2>, dim3(M), dim3(512), 0, st, a);
-  else hipLaunchKernelGGL(row_norm_kernel<4>, dim3(M), dim3(512), 0, st, a);
+  if (cpt <= 1) hipLaunchKernelGGL(row_norm_kernel<1>, dim3(M), dim3(512), lds, st, a);
+  else if (cpt <= 2) hipLaunchKernelGGL(row_norm_kernel<2>, dim3(M), dim3(512), lds, st, a);
+  else hipLaunchKernelGGL(row_norm_kernel<4>, dim3(M), dim3(512), lds, st, a);
   return check_launch();
 }
 

@@ -425,14 +425,41 @@ __global__ __launch_bounds__(256) void sb_attn_kernel(SbAttnArgs a) {
   const int ntot = (a.N + 2 * a.Kh) * H;
   const uint16_t* row = a.qkv + (size_t)b * ntot;
   const float* tab = a.rope_tab + (size_t)b * half * 2;
-  // rotate the G query heads (f32 throughout, one cast: llama3/model.py:249-270)
-  for (int e = tid; e < G * half; e += 256) {
-    const int g = e / half, i = e - g * half;
+  // Per-head RMSNorm (Qwen3 q_norm / k_norm: f32 with one cast, qwen3/model.py:478-484) of a head vector held as
+  // one (x1, x2) pair per lane by `half` consecutive lanes, then the rotation: f32 throughout with one cast for
+  // Llama3 (llama3/model.py:249-270); sin / cos and every product rounded to bf16 for Qwen3 (qwen3/model.py:432-453).
+  const bool qwen = a.family == TMX_FAMILY_QWEN3;
+  auto norm_rotate = [&](float x1, float x2, const uint16_t* nw, int i, float& o1, float& o2) __attribute__((always_inline)) {
+    if (nw) {
+      float ss = x1 * x1 + x2 * x2;
+#pragma unroll
+      for (int off = half / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      const float rms = sqrtf(ss / (float)H + a.eps);
+      x1 = rbf(bf2f(nw[i]) * (x1 / rms));
+      x2 = rbf(bf2f(nw[i + half]) * (x2 / rms));
+    }
+    float sn = tab[i * 2], cs = tab[i * 2 + 1];
+    if (qwen) {
+      sn = rbf(sn);
+      cs = rbf(cs);
+      o1 = rbf(x1 * cs) - rbf(x2 * sn);
+      o2 = rbf(x2 * cs) + rbf(x1 * sn);
+    } else {
+      o1 = x1 * cs - x2 * sn;
+      o2 = x2 * cs + x1 * sn;
+    }
+  };
+  static_assert(G * (H / 2) <= 256, "one (x1, x2) pair of the query heads per thread");
+  {  // the G query heads: thread (g, i); the `half` lanes of a head are consecutive and aligned
+    const bool act = tid < G * half;
+    const int g = act ? tid / half : 0, i = tid % half;
     const uint16_t* qh = row + (size_t)(kvh * G + g) * H;
-    const float x1 = bf2f(qh[i]), x2 = bf2f(qh[i + half]);
-    const float sn = tab[i * 2], cs = tab[i * 2 + 1];
-    q_s[g][i] = f2bf(x1 * cs - x2 * sn);
-    q_s[g][i + half] = f2bf(x2 * cs + x1 * sn);
+    float o1, o2;
+    norm_rotate(act ? bf2f(qh[i]) : 0.f, act ? bf2f(qh[i + half]) : 0.f, a.q_norm_w, i, o1, o2);
+    if (act) {
+      q_s[g][i] = f2bf(o1);
+      q_s[g][i + half] = f2bf(o2);
+    }
   }
   uint16_t* kc = a.kcache + ((size_t)b * a.C * a.Kh + kvh) * H;
   uint16_t* vc = a.vcache + ((size_t)b * a.C * a.Kh + kvh) * H;
@@ -441,10 +468,10 @@ __global__ __launch_bounds__(256) void sb_attn_kernel(SbAttnArgs a) {
     const int slot = step % a.C;
     if (tid < half) {
       const uint16_t* kh = row + (size_t)(a.N + kvh) * H;
-      const float x1 = bf2f(kh[tid]), x2 = bf2f(kh[tid + half]);
-      const float sn = tab[tid * 2], cs = tab[tid * 2 + 1];
-      kc[(size_t)slot * row_stride + tid] = f2bf(x1 * cs - x2 * sn);
-      kc[(size_t)slot * row_stride + tid + half] = f2bf(x2 * cs + x1 * sn);
+      float o1, o2;
+      norm_rotate(bf2f(kh[tid]), bf2f(kh[tid + half]), a.k_norm_w, tid, o1, o2);
+      kc[(size_t)slot * row_stride + tid] = f2bf(o1);
+      kc[(size_t)slot * row_stride + tid + half] = f2bf(o2);
     } else if (tid >= 128 && tid < 128 + H) {
       vc[(size_t)slot * row_stride + (tid - 128)] = row[(size_t)(a.N + a.Kh + kvh) * H + (tid - 128)];
     }

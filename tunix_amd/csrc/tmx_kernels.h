@@ -119,6 +119,7 @@ struct RowNormArgs {
   int D;
   float eps;
   int family;
+  RouterArgs router;            // router.w != null: the row's workgroup also routes the token from xn (MoE layers)
 };
 
 struct RopeArgs {
@@ -260,6 +261,10 @@ struct SbAttnArgs {
   float* partial;           // [B][Kh][nsplit][G][H + 2]
   int B, N, Kh, C, nsplit;
   float scale;
+  const uint16_t* q_norm_w;  // [H] per-head RMSNorm of q and k before the rotation (Qwen3), or null
+  const uint16_t* k_norm_w;
+  float eps;
+  int family;                // rotation rounding: TMX_FAMILY_*
 };
 
 int sb_linear(hipStream_t st, const SbLinearArgs& a, int pro, int epi);  // pro: 0 plain, 1 norm, 2 attention merge; epi: 0 plain, 1 residual, 2 SwiGLU
