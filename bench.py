@@ -524,11 +524,12 @@ def main():
     sampler.share_prompt_kv = True
     lib = _lib.lib()
     st = fresh_state()
-    sampler.run_steps(st, args.warmup, sample=True)
+    n_prof = min(8, args.steps)
+    # at the middle of the timed window: the mean context, where the unshared replay's mean sits too
+    sampler.run_steps(st, args.warmup + (args.steps - n_prof) // 2, sample=True)
     ms = np.zeros(len(CLASS_NAMES), np.float32)
     cnt = np.zeros(len(CLASS_NAMES), np.int32)
     tot = 0.0
-    n_prof = min(8, args.steps)
     for _ in range(n_prof):
       cs = sampler._c_state(st)
       rc = lib.tmx_decode_steps_profiled(ctypes.byref(model.desc()), ctypes.byref(cs), _lib.stream(), 1, 1,
