@@ -227,8 +227,8 @@ int tmx_gqa_decode_attention(void* stream, const void* q, const void* kcache, co
  * first sequence, for all of the group's queries; every sequence reads only its own slots from share_len
  * on.  The softmax runs over the same positions as in tmx_gqa_decode_attention (the results differ in
  * the order of the f32 sums only).  The caller vouches for the sharing; nothing checks that the rows
- * really are equal.  B <= 128, B % share_group == 0, share_len >= 32, H in {64, 128}, N / Kh in
- * {1, 2, 4}, else TMX_ERR_UNSUPPORTED.  workspace: tmx_gqa_decode_shared_workspace_bytes() bytes. */
+ * really are equal.  B <= 128, B % share_group == 0, 32 <= share_len <= C, H in {64, 128}, N / Kh in
+ * {1, 2, 4, 8}, else TMX_ERR_UNSUPPORTED.  workspace: tmx_gqa_decode_shared_workspace_bytes() bytes. */
 size_t tmx_gqa_decode_shared_workspace_bytes(int B, int N, int Kh, int H, int C);
 int tmx_gqa_decode_attention_shared(void* stream, const void* q, const void* kcache, const void* vcache,
                                     const uint8_t* input_mask, const int32_t* step, int buf_len, void* out,

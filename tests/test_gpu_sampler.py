@@ -481,25 +481,34 @@ def test_moe_decoder_matches_oracle():
   _compare_greedy(out, ref, 4, min_checked=20, lp_extra=2.0 ** -7)
 
 
-@pytest.mark.parametrize('nseq,top_p', [(4, 1.0), (150, 1.0), (6, 0.8), (70, 0.9)])
-def test_graph_replay_matches_plain_launches_on_every_replay(nseq, top_p):
+@pytest.mark.parametrize('nseq,top_p,group', [(4, 1.0, 1), (150, 1.0, 1), (6, 0.8, 1), (70, 0.9, 1), (16, 1.0, 4),
+                                               (16, 1.0, 8)])
+def test_graph_replay_matches_plain_launches_on_every_replay(nseq, top_p, group):
   """tmx_decode_steps_graph against tmx_decode_steps: several graph calls in a row, with the
   program's own eager work (a plain step, host reads) and synchronisation between them; every
   call's tokens, logprobs, KV cache and step counter equal the plain launches'.  4 sequences: the
   small-batch launches; 150: the many-rows kernels; top_p < 1: the selection launches of the
   top-p branch (6 sequences behind the 64-row head and the gate|up hand-over, 70 behind the head in
-  256 x 256 blocks) are recorded and replayed."""
-  cfg = C.TOY
+  256 x 256 blocks) are recorded and replayed.  group > 1: four rows per 40-token prompt on a model with
+  that many query heads per KV head, so the recorded attention launches are the ones that read the common
+  prompt slots once per group of rows (vector walk plus merge for 4 heads per KV head, the walk on the
+  matrix pipe for 8)."""
+  cfg = C.TOY if group == 1 else OM.Config('llama3', 2, 1024, 256, 1024, 8, 64, 8 // group, rope_theta=10000,
+                                           norm_eps=1e-5, tied=False)
   _, model = _pair(cfg, seed=17, targets=('q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj'))
   rng = np.random.default_rng(2)
-  ids = np.stack([rng.integers(3, cfg.vocab_size, 8) for _ in range(nseq)]).astype(np.int32)
+  plen = 8 if group == 1 else 40
+  rows = 1 if group == 1 else 4
+  base = [rng.integers(3, cfg.vocab_size, plen) for _ in range(nseq // rows)]
+  ids = np.stack([base[i // rows] for i in range(nseq)]).astype(np.int32)
   def run(graph):
-    s = _sampler(model, cfg, 64)
+    s = _sampler(model, cfg, plen + 56)
     s.eos_ids = np.array([-1])
-    st = s.init_sample_state(ids, 64, False, None, 0.9, top_p, None, 5, include_logprobs=True,
-                             prompt_lengths=np.full(nseq, 8))
+    st = s.init_sample_state(ids, plen + 56, False, None, 0.9, top_p, None, 5, include_logprobs=True,
+                             prompt_lengths=np.full(nseq, plen))
+    assert st['share_group'] == rows
     snaps = []
-    s.run_steps(st, 7, sample=False, graph=graph)
+    s.run_steps(st, plen - 1, sample=False, graph=graph)
     for n in (9, 1, 12, 5, 16):
       s.run_steps(st, n, sample=True, graph=graph)
       torch.cuda.synchronize()
