@@ -262,6 +262,18 @@ int tmx_head_sample(void* stream, const void* x, const void* head_w, int M, int 
                     int32_t* token_buffer, float* logprobs, uint8_t* done, int buf_len,
                     float* logits_out, void* workspace);
 
+/* The same from a copy of the head matrix laid out for streaming: tmx_head_tiles_pack writes head_tiles
+ * (V * D bf16 elements, like head_w) from head_w[V, D]; 32 rows x 64 columns form a tile of 4 KiB, the tiles of
+ * 32 rows follow each other along D, and inside a tile the 16 bytes head_w[32 vt + n][64 kt + 32 h + 8 t .. + 7]
+ * sit at byte (t * 64 + 32 h + n) * 16.  V % 32 == 0, D % 64 == 0, V <= 32 * 65535.  The layout has no counterpart
+ * in the reference (jnp arrays are row-major); results are bit-identical to tmx_head_sample's. */
+int tmx_head_tiles_pack(void* stream, const void* head_w, void* head_tiles, int V, int D);
+int tmx_head_sample_tiles(void* stream, const void* x, const void* head_tiles, int M, int D, int V, int mode,
+                          float temperature, uint32_t seed_hi, uint32_t seed_lo, const int32_t* step,
+                          const int32_t* forbidden, int n_forbidden, const int32_t* eos, int n_eos,
+                          int32_t* token_buffer, float* logprobs, uint8_t* done, int buf_len,
+                          float* logits_out, void* workspace);
+
 /* The sorting branch of sample_top_p (top_p < 1 and / or top_k > 0),
  * tunix/generate/sampler.py:136-153: candidates = the top_k (or all V) logits in descending
  * order, ties in index order; probs = softmax over the candidates; a candidate is dropped when
@@ -334,6 +346,9 @@ typedef struct {
   const void* final_norm_w; /* bf16 [D] */
   const void* head;         /* bf16 [V, D]: the embedding table when tied, else lm_head^T */
   const tmx_layer_desc* layers; /* HOST array of num_layers entries */
+  const void* head_tiles;   /* NULL, or the head matrix once more in the layout tmx_head_tiles_pack writes (V % 32
+                               == 0, D % 64 == 0): steps of up to 64 sequences then stream that copy, every byte
+                               in whole cache lines (the 1.05 GB head of the 8B shape: 190 us against 252 us) */
 } tmx_model_desc;
 
 /* Mirrors _SamplingState (tunix/generate/sampler.py:53-109); all arrays on the device. */

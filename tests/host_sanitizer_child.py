@@ -62,7 +62,7 @@ def model_desc(family, layers, vocab, dm, f, n, kh, h, experts, per_tok, group, 
 def main():
   lib = _lib.lib()
   assert os.path.basename(_lib.LIB_PATH) == 'libtmx_hostsan.so', _lib.LIB_PATH
-  assert lib.tmx_abi_version() >= 6
+  assert lib.tmx_abi_version() >= 7
   sizes = []
   for name, c in CONFIGS.items():
     d, keep = model_desc(*c)

@@ -474,6 +474,48 @@ def _head_inputs(M, D, V, seed):
   return x, w
 
 
+def head_tiles_layout(w):
+  """The streaming copy of a head matrix, restated from the C header: tiles of 32 rows x 64 columns, the
+  tiles of a row block one after the other; inside a tile the 8 elements w[32 vt + n, 64 kt + 32 h + 8 t : + 8]
+  at element (t * 64 + 32 h + n) * 8.  Plain loops over the pieces."""
+  V, D = w.shape
+  out = np.empty(V * D, w.dtype)
+  for vt in range(V // 32):
+    for kt in range(D // 64):
+      base = (vt * (D // 64) + kt) * 2048
+      for t in range(4):
+        for h in range(2):
+          for n in range(32):
+            k0 = 64 * kt + 32 * h + 8 * t
+            out[base + (t * 64 + 32 * h + n) * 8: base + (t * 64 + 32 * h + n) * 8 + 8] = w[32 * vt + n, k0:k0 + 8]
+  return out
+
+
+def test_head_tiles_pack_writes_the_documented_layout():
+  T = G.Keep()
+  V, D = 96, 192
+  w = bf16_round(np.random.default_rng(3).standard_normal((V, D)).astype(np.float32))
+  tiles = torch.zeros(V * D, dtype=torch.bfloat16, device=G.DEV)
+  G.call('tmx_head_tiles_pack', S(), T.bf(w), G.p(tiles), V, D)
+  G.sync()
+  np.testing.assert_array_equal(tiles.float().cpu().numpy(), head_tiles_layout(w))
+  # shapes the layout does not cover are refused before anything is launched
+  lib = _lib.lib()
+  assert lib.tmx_head_tiles_pack(S(), T.bf(w), G.p(tiles), 80, 192) != 0
+  assert lib.tmx_head_tiles_pack(S(), T.bf(w), G.p(tiles), 96, 96) != 0
+
+
+HEAD_LAYOUT = 'rows'  # 'tiles': _run_head hands the kernel the streaming copy (tmx_head_sample_tiles)
+
+
+@pytest.fixture(params=['rows', 'tiles'])
+def head_layout(request):
+  global HEAD_LAYOUT
+  HEAD_LAYOUT = request.param
+  yield request.param
+  HEAD_LAYOUT = 'rows'
+
+
 def _run_head(x, w, mode, temperature, key, step, forbidden=(), eos=(-1,), col_len=20):
   T = G.Keep()
   M, D = x.shape
@@ -485,15 +527,35 @@ def _run_head(x, w, mode, temperature, key, step, forbidden=(), eos=(-1,), col_l
   done = torch.zeros(M, dtype=torch.uint8, device=G.DEV)
   logits = torch.empty(M, V, dtype=torch.float32, device=G.DEV)
   fb = T.i32(list(forbidden)) if forbidden else None
-  G.call('tmx_head_sample', S(), T.bf(x), T.bf(w), M, D, V, mode, temperature, int(key[0]), int(key[1]),
+  entry, wd = 'tmx_head_sample', T.bf(w)
+  if HEAD_LAYOUT == 'tiles':
+    tiles = torch.empty(V * D, dtype=torch.bfloat16, device=G.DEV)
+    G.call('tmx_head_tiles_pack', S(), wd, G.p(tiles), V, D)
+    entry, wd = 'tmx_head_sample_tiles', G.p(tiles)
+  G.call(entry, S(), T.bf(x), wd, M, D, V, mode, temperature, int(key[0]), int(key[1]),
          T.i32([step]), fb, len(forbidden), T.i32(list(eos)), len(eos), G.p(tok), G.p(lp),
          G.p(done), col_len, G.p(logits), G.p(ws))
   G.sync()
   return tok.cpu().numpy(), lp.cpu().numpy(), done.cpu().numpy(), logits.cpu().numpy()
 
 
+@pytest.mark.parametrize('M,D,V', [(1, 256, 1024), (40, 320, 2080), (64, 4096, 1024)])
+def test_head_from_tiles_equals_head_from_rows_bit_for_bit(M, D, V):
+  """Both layouts feed the same 16-byte pieces to the same matrix instructions in the same order: logits,
+  tokens and log-probs are identical, greedy and sampled."""
+  global HEAD_LAYOUT
+  x, w = _head_inputs(M, D, V, 3 * M + V)
+  for mode, temp, key in ((0, 1.0, (0, 0)), (1, 0.7, prng.prng_key(4))):
+    outs = {}
+    for HEAD_LAYOUT in ('rows', 'tiles'):
+      outs[HEAD_LAYOUT] = _run_head(x, w, mode, temp, key, 2)
+    HEAD_LAYOUT = 'rows'
+    for a, b in zip(outs['rows'], outs['tiles']):
+      np.testing.assert_array_equal(a, b)
+
+
 @pytest.mark.parametrize('M,D,V', [(1, 256, 1024), (5, 512, 4096), (64, 256, 1056), (100, 128, 2048)])
-def test_head_greedy(M, D, V):
+def test_head_greedy(M, D, V, head_layout):
   T = G.Keep()
   x, w = _head_inputs(M, D, V, M + V)
   step = 3
@@ -554,7 +616,7 @@ def test_head_scoring_clips_logits_like_the_reference():
   # (checked on the last column's neighbours through the closed form of the oracle pin)
 
 
-def test_head_greedy_ties_pick_first_index_and_forbidden():
+def test_head_greedy_ties_pick_first_index_and_forbidden(head_layout):
   T = G.Keep()
   M, D, V = 3, 128, 1024
   x, w = _head_inputs(M, D, V, 5)
@@ -571,7 +633,7 @@ def test_head_greedy_ties_pick_first_index_and_forbidden():
 
 
 @pytest.mark.parametrize('M,D,V,temp', [(4, 256, 1024, 0.9), (64, 128, 4096, 1.0), (33, 256, 2080, 0.7)])
-def test_head_temperature_sampling_matches_threefry_oracle(M, D, V, temp):
+def test_head_temperature_sampling_matches_threefry_oracle(M, D, V, temp, head_layout):
   T = G.Keep()
   x, w = _head_inputs(M, D, V, V + 1)
   seed_key = prng.prng_key(1234)

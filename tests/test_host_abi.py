@@ -51,7 +51,7 @@ def test_header_is_plain_c_and_cxx():
 
 def test_status_strings_and_version():
   lib = _lib.lib()
-  assert lib.tmx_abi_version() == 6
+  assert lib.tmx_abi_version() == 7
   assert lib.tmx_status_string(0) == b'ok'
   for code in (-1, -2, -3, -4):
     assert len(lib.tmx_status_string(code)) > 5

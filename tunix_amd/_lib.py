@@ -36,6 +36,9 @@ SIGNATURES = {
     'tmx_gqa_attention_rows': [vp, vp, vp, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, ci, ci],
     'tmx_head_sample': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
                         vp, vp],
+    'tmx_head_sample_tiles': [vp, vp, vp, ci, ci, ci, ci, cf, cu32, cu32, vp, vp, ci, vp, ci, vp, vp, vp, ci,
+                              vp, vp],
+    'tmx_head_tiles_pack': [vp, vp, vp, ci, ci],
     'tmx_head_sample_nucleus': [vp, vp, vp, ci, ci, ci, cf, cf, ci, cu32, cu32, vp, vp, ci, vp, ci, vp, vp,
                                 vp, ci, vp, vp, ctypes.c_size_t],
     'tmx_moe_route': [vp, vp, vp, ci, ci, ci, ci, vp, vp],

@@ -534,6 +534,7 @@ static int decode_steps_impl(const tmx_model_desc* m, const tmx_decode_state* s,
       HeadArgs a = {};
       a.x = w.xn;
       a.w = (const uint16_t*)m->head;
+      a.w_tiles = (const uint16_t*)m->head_tiles;
       a.M = B; a.D = D; a.V = m->vocab_size;
       a.mode = s->sampling_mode;
       a.temperature = s->temperature;

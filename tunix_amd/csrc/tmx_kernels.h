@@ -174,6 +174,7 @@ struct AttnArgs {
 struct HeadArgs {
   const uint16_t* x;  // [M, D] final-normed hidden states
   const uint16_t* w;  // [V, D]
+  const uint16_t* w_tiles;  // the same matrix in the tile layout of head_tiles_kernel, or null
   int M, D, V;
   int mode;
   float temperature;

@@ -92,7 +92,7 @@ class ModelDesc(ctypes.Structure):
               ('num_kv_heads', ctypes.c_int), ('head_dim', ctypes.c_int), ('num_experts', ctypes.c_int),
               ('experts_per_tok', ctypes.c_int), ('rope_theta', ctypes.c_float),
               ('norm_eps', ctypes.c_float), ('embed', ctypes.c_void_p), ('final_norm_w', ctypes.c_void_p),
-              ('head', ctypes.c_void_p), ('layers', ctypes.POINTER(LayerDesc))]
+              ('head', ctypes.c_void_p), ('layers', ctypes.POINTER(LayerDesc)), ('head_tiles', ctypes.c_void_p)]
 
 
 class DecodeState(ctypes.Structure):
@@ -135,6 +135,8 @@ class QLoRAModel:
     self.layers = []          # list of dict name -> tensor / PackedLinear
     self.embed = None         # bf16 [V, D]
     self.head = None          # bf16 [V, D] (is self.embed when tied)
+    self.head_tiles = None    # the head once more in the streaming layout (tmx_head_tiles_pack), made by desc()
+    self.stream_head = True   # False: decode steps read the row-major head
     self.final_norm = None
     self.lora_rank = 0
     self.lora_alpha = 0.0
@@ -364,6 +366,13 @@ class QLoRAModel:
     d.num_experts, d.experts_per_tok = c.num_experts or 0, c.num_experts_per_tok or 0
     d.rope_theta, d.norm_eps = float(c.rope_theta), float(c.norm_eps)
     d.embed, d.final_norm_w, d.head = self.embed.data_ptr(), self.final_norm.data_ptr(), self.head.data_ptr()
+    if self.stream_head and c.vocab_size % 32 == 0 and c.embed_dim % 64 == 0 and c.vocab_size <= 32 * 65535:
+      # one more copy of the head (V * D * 2 bytes) that one-token steps of up to 64 sequences stream
+      if self.head_tiles is None:
+        self.head_tiles = torch.empty_like(self.head)
+        _lib.check(_lib.lib().tmx_head_tiles_pack(_lib.stream(), _lib.ptr(self.head), _lib.ptr(self.head_tiles),
+                                                  c.vocab_size, c.embed_dim), 'tmx_head_tiles_pack')
+      d.head_tiles = self.head_tiles.data_ptr()
     d.layers = ctypes.cast(arr, ctypes.POINTER(LayerDesc))
     self._desc, self._keep = d, arr
     return d
