@@ -432,7 +432,7 @@ def main():
     symbols.update({
         # more than 64 rows: the head in 256 x 256 blocks (template argument: the sampling mode, 1 = top-p branch);
         # with top_p < 1 the class also holds the three selection launches of nucleus.hip
-        ('tmx::head_wide_kernel<1>' if batch > 64 else f'tmx::head_kernel<{min(mt, 2)}>'): ['head_sample'],
+        ('tmx::head_wide_kernel<1>' if batch > 64 else f'tmx::head_kernel<{min(mt, 2)}, true>'): ['head_sample'],
     })
     idx = {n: i for i, n in enumerate(CLASS_NAMES)}
     # An event pair around a launch also times the packet processing on both sides of it, so it

@@ -784,7 +784,8 @@ def test_head_sampling_distribution_chi2():
 
 # ---- routed experts (Qwen3 MoE) ---------------------------------------------------------------
 
-@pytest.mark.parametrize('B,D,E,k', [(8, 256, 16, 4), (32, 512, 128, 8), (3, 256, 8, 1), (32, 2048, 128, 8)])
+@pytest.mark.parametrize('B,D,E,k', [(8, 256, 16, 4), (32, 512, 128, 8), (3, 256, 8, 1), (32, 2048, 128, 8),
+                                     (12, 2304, 160, 16), (5, 128, 32, 32)])
 def test_moe_route_matches_oracle(B, D, E, k):
   T = G.Keep()
   rng = np.random.default_rng(B + E)

@@ -169,7 +169,7 @@ __device__ __forceinline__ void add_lora8(float* o, const float* t_s, const uint
 // In embedding mode it also fills this step's RoPE sin/cos table row.
 template <int CPT>  // 8-element chunks per thread, D <= 4096 * CPT
 __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
-  extern __shared__ float route_sm[];  // moe_router_lds_floats(D, E) floats when the row is routed here, else none
+  extern __shared__ __align__(16) float route_sm[];  // moe_router_lds_floats(D, E) floats when the row is routed here, else none
   __shared__ float smem[8];
   __shared__ float t_s[TMX_MAX_RPAD];
   __shared__ float t_stage[TMX_MAX_LORA_SPLITS * 64];
@@ -236,13 +236,26 @@ __global__ __launch_bounds__(512) void row_norm_kernel(RowNormArgs a) {
         unpack8(*reinterpret_cast<const uint4*>(src + n0), v[i]);
       } else if (a.moe_y) {
         // bf16(sum over the token's experts of weight * expert output), f32 accumulation
-        for (int j = 0; j < a.top_k; ++j) {
-          float y8[8];
-          const size_t p = (size_t)m * a.top_k + j;
-          unpack8(*reinterpret_cast<const uint4*>(a.moe_y + p * a.D + n0), y8);
-          const float w = a.moe_w[p];
+        // (eight experts' rows and weights are requested together: one memory round trip per eight, in the
+        // experts' order)
+        for (int j0 = 0; j0 < a.top_k; j0 += 8) {
+          uint4 yr[8];
+          float wr[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[i][e] = fmaf(w, y8[e], v[i][e]);
+          for (int u = 0; u < 8; ++u) {
+            const size_t p = (size_t)m * a.top_k + min(j0 + u, a.top_k - 1);
+            yr[u] = *reinterpret_cast<const uint4*>(a.moe_y + p * a.D + n0);
+            wr[u] = j0 + u < a.top_k ? a.moe_w[p] : 0.f;
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            if (j0 + u < a.top_k) {
+              float y8[8];
+              unpack8(yr[u], y8);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[i][e] = fmaf(wr[u], y8[e], v[i][e]);
+            }
+          }
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[i][e] = rbf(v[i][e]);

@@ -12,7 +12,7 @@
 namespace tmx {
 
 __global__ __launch_bounds__(kRouterThreads) void moe_router_kernel(RouterArgs a) {
-  extern __shared__ float sm[];
+  extern __shared__ __align__(16) float sm[];
   const int b = blockIdx.x;
   for (int d = threadIdx.x; d < a.D; d += kRouterThreads) sm[d] = bf2f(a.x[(size_t)b * a.D + d]);
   __syncthreads();
@@ -21,7 +21,7 @@ __global__ __launch_bounds__(kRouterThreads) void moe_router_kernel(RouterArgs a
 
 int moe_route(hipStream_t st, const RouterArgs& a, int B) {
   if (!a.x || !a.w || !a.expert_of || !a.weight_of) return TMX_ERR_ARG;
-  if (B <= 0 || a.D <= 0 || a.E <= 0 || a.E % 8 || a.top_k <= 0 || a.top_k > 64 || a.top_k > a.E)
+  if (B <= 0 || a.D <= 0 || a.D % 4 || a.E <= 0 || a.E % 8 || a.top_k <= 0 || a.top_k > 64 || a.top_k > a.E)
     return TMX_ERR_SHAPE;
   const size_t lds = moe_router_lds_floats(a.D, a.E) * sizeof(float);
   if (lds > 60000) return TMX_ERR_SHAPE;
