@@ -190,13 +190,33 @@ __global__ __launch_bounds__(H) void gqa_combine_kernel(AttnArgs a) {
   const int nparts = a.nsplit + a.psplits;
   const float* pr = a.partial + (((size_t)b * a.Kh + kvh) * nparts * G + g) * (H + 2);
   const size_t sstride = (size_t)G * (H + 2);
-  float mm = -1e30f;
-  for (int s = 0; s < nparts; ++s) mm = fmaxf(mm, pr[s * sstride + H]);
-  float ls = 0.f, o = 0.f;
-  for (int s = 0; s < nparts; ++s) {
-    const float w = __expf(pr[s * sstride + H] - mm);
-    ls += pr[s * sstride + H + 1] * w;
-    o += pr[s * sstride + d] * w;
+  // the parts are requested eight at a time (clamped indices), so that a row costs one memory round trip and not
+  // one per part; merged in ascending order
+  float mm = -1e30f, ls = 0.f, o = 0.f;
+  for (int s0 = 0; s0 < nparts; s0 += 8) {
+    float pm[8], pl[8], po[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float* q = pr + (size_t)min(s0 + u, nparts - 1) * sstride;
+      pm[u] = s0 + u < nparts ? q[H] : -1e30f;
+      pl[u] = q[H + 1];
+      po[u] = q[d];
+    }
+    float mn = mm;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) mn = fmaxf(mn, pm[u]);
+    const float alpha = __expf(mm - mn);
+    ls *= alpha;
+    o *= alpha;
+    mm = mn;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (s0 + u < nparts) {
+        const float w = __expf(pm[u] - mm);
+        ls += pl[u] * w;
+        o += po[u] * w;
+      }
+    }
   }
   a.out[((size_t)b * a.N + kvh * G + g) * H + d] = f2bf(ls > 0.f ? o / ls : 0.f);
 }
