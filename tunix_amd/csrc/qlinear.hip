@@ -9,7 +9,8 @@
 // packed tile format stores, for every 64(k) x 32(n) tile, the 32 nibbles a lane
 // needs as ONE 128-bit word, so a wave fetches a tile with a single coalesced
 // 1 KiB load and never touches LDS for weights.  Nibbles are widened with
-// v_cvt_f32_ubyteN, scaled with one fma ((u - 8) * s is exact in f32) and
+// v_cvt_f32_ubyteN (or two at a time with v_cvt_pk_f32_fp8: dequant_word in tmx_common.h),
+// scaled with one fma ((u - 8) * s is exact in f32) and
 // rounded pairwise to bf16 by the hardware converter, which reproduces the
 // reference's bf16 dequantised weight bit for bit before it enters the MFMA.
 #include <atomic>
@@ -452,7 +453,7 @@ __global__ __launch_bounds__(256, 2) void moe_stream_kernel(MoeArgs m) {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
               acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, xq[sl & 1][t]),
-                                                               dequant_word(wd[t], s_c[c], m8s), acc[c], 0, 0, 0);
+                                                               dequant_word<true>(wd[t], s_c[c], m8s), acc[c], 0, 0, 0);
           }
         });
       }
@@ -996,7 +997,7 @@ __global__ __launch_bounds__(512, 1) void qlinear_gate_up8_kernel(QLinearArgs a)
     const uint32_t wd[4] = {wc.x, wc.y, wc.z, wc.w};
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const bf16x8_t b = dequant_word(wd[t], s_c, m8s);
+      const bf16x8_t b = dequant_word<true>(wd[t], s_c, m8s);
 #pragma unroll
       for (int m = 0; m < MT; ++m)
         acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[m][t], b, acc[m], 0, 0, 0);
@@ -2098,7 +2099,7 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(const uint4* qw, cons
   const uint32_t wd[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    const bf16x8_t b = dequant_word(wd[t], s, -8.f * s);
+    const bf16x8_t b = dequant_word<true>(wd[t], s, -8.f * s);
     uint16_t e[8];
     __builtin_memcpy(e, &b, 16);
 #pragma unroll

@@ -268,7 +268,7 @@ __global__ __launch_bounds__(kSbThreads) void sb_linear_kernel(SbLinearArgs a) {
         }
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[t], dequant_word(wd[t], sc, m8s), acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[t], dequant_word<true>(wd[t], sc, m8s), acc, 0, 0, 0);
         if (mine(base + i)) {
 #pragma unroll
           for (int q = 0; q < 2; ++q) {

@@ -92,28 +92,57 @@ __device__ __forceinline__ void dequant_masks(uint32_t d, uint32_t& lo, uint32_t
 template <int P>
 __device__ __forceinline__ uint32_t dequant_part(uint32_t lo, uint32_t hi, float s, float m8s);
 
+// A byte 0x0U read as an fp8 number (E4M3, bias 7) is U * 2^-9 for every U in 0..15: below 8 it is subnormal
+// (U / 8 * 2^-6), from 8 on its exponent field is 1 ((1 + (U - 8) / 8) * 2^-6).  So one v_cvt_pk_f32_fp8 widens
+// two nibbles of a masked word at once, where v_cvt_f32_ubyteN takes one instruction per nibble; the factor
+// 2^9 goes into the scale (exact).  w: a word of four bytes 0x0U; returns the floats of bytes (0, 1) or (2, 3).
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+template <bool HIGH>
+__device__ __forceinline__ f32x2_t nibble_pair_f32(uint32_t w) {
+  return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, HIGH);
+}
+constexpr float kNibbleUnit = 512.f;  // 1 / (2^-9)
+
 // Expand one 32-bit word (8 nibbles, element j = 2 (i % 4) + i / 4 for nibble i)
 // into the 8 bf16 B-operand values of one MFMA step: bf16((u - 8) * s).
+// PAIRS = false: fma(u, s, -8 s) with u widened by v_cvt_f32_ubyteN, one instruction per nibble.
+// PAIRS = true: fma(u * 2^-9, s * 2^9, -8 s) with two nibbles widened per v_cvt_pk_f32_fp8 (19 instead of 23
+// instructions per word).  Both are (u - 8) * s exactly (4 + 8 significant bits), rounded once to bf16.  The pair
+// form pays where the loop is bound by these instructions (the fused gate|up launch -3 %, the expert stream -2 %,
+// the 1..4-row projections -2 % of their step);
+// in the loops bound by the matrix pipe it measured slower (128-row projections +1.6 % on the step), so they
+// keep the byte form.
+template <bool PAIRS = false>
 __device__ __forceinline__ bf16x8_t dequant_word(uint32_t d, float s, float m8s) {
   uint32_t lo = d & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
   uint32_t hi = (d >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7 in bytes 0..3
-  // keep the two masked words opaque so that each byte is widened by one
-  // v_cvt_f32_ubyteN instead of a bit-field extract plus a conversion
-  asm volatile("" : "+v"(lo), "+v"(hi));
-  // nibble i: byte i/2 of (i even ? lo : hi)
-  const float n0 = (float)(lo & 0xFF), n1 = (float)(hi & 0xFF);
-  const float n2 = (float)((lo >> 8) & 0xFF), n3 = (float)((hi >> 8) & 0xFF);
-  const float n4 = (float)((lo >> 16) & 0xFF), n5 = (float)((hi >> 16) & 0xFF);
-  const float n6 = (float)(lo >> 24), n7 = (float)(hi >> 24);
   // register p holds elements j = 2p, 2p + 1  <->  nibbles p, p + 4
   uint32_t p[4];
-  p[0] = pack_bf2(fmaf(n0, s, m8s), fmaf(n4, s, m8s));
-  p[1] = pack_bf2(fmaf(n1, s, m8s), fmaf(n5, s, m8s));
-  p[2] = pack_bf2(fmaf(n2, s, m8s), fmaf(n6, s, m8s));
-  p[3] = pack_bf2(fmaf(n3, s, m8s), fmaf(n7, s, m8s));
-  bf16x8_t b;
-  __builtin_memcpy(&b, p, 16);
-  return b;
+  if constexpr (PAIRS) {
+    const float s9 = s * kNibbleUnit;
+    const f32x2_t a = nibble_pair_f32<false>(lo), b = nibble_pair_f32<true>(lo);  // nibbles (0, 2), (4, 6)
+    const f32x2_t c = nibble_pair_f32<false>(hi), e = nibble_pair_f32<true>(hi);  // nibbles (1, 3), (5, 7)
+    p[0] = pack_bf2(fmaf(a.x, s9, m8s), fmaf(b.x, s9, m8s));
+    p[1] = pack_bf2(fmaf(c.x, s9, m8s), fmaf(e.x, s9, m8s));
+    p[2] = pack_bf2(fmaf(a.y, s9, m8s), fmaf(b.y, s9, m8s));
+    p[3] = pack_bf2(fmaf(c.y, s9, m8s), fmaf(e.y, s9, m8s));
+  } else {
+    // keep the two masked words opaque so that each byte is widened by one
+    // v_cvt_f32_ubyteN instead of a bit-field extract plus a conversion
+    asm volatile("" : "+v"(lo), "+v"(hi));
+    // nibble i: byte i/2 of (i even ? lo : hi)
+    const float n0 = (float)(lo & 0xFF), n1 = (float)(hi & 0xFF);
+    const float n2 = (float)((lo >> 8) & 0xFF), n3 = (float)((hi >> 8) & 0xFF);
+    const float n4 = (float)((lo >> 16) & 0xFF), n5 = (float)((hi >> 16) & 0xFF);
+    const float n6 = (float)(lo >> 24), n7 = (float)(hi >> 24);
+    p[0] = pack_bf2(fmaf(n0, s, m8s), fmaf(n4, s, m8s));
+    p[1] = pack_bf2(fmaf(n1, s, m8s), fmaf(n5, s, m8s));
+    p[2] = pack_bf2(fmaf(n2, s, m8s), fmaf(n6, s, m8s));
+    p[3] = pack_bf2(fmaf(n3, s, m8s), fmaf(n7, s, m8s));
+  }
+  bf16x8_t r;
+  __builtin_memcpy(&r, p, 16);
+  return r;
 }
 
 template <int P>
