@@ -343,7 +343,9 @@ def test_host_code_under_address_and_undefined_sanitizers():
   newest = max(newest, os.path.getmtime(os.path.join(os.path.dirname(tb.CSRC), '..', 'include', 'tmx.h')))
   if not os.path.exists(tb.HOSTSAN_LIB_PATH) or os.path.getmtime(tb.HOSTSAN_LIB_PATH) < newest:
     tb.build(host_sanitizers=True)
-  env = dict(os.environ, TMX_LIB=tb.HOSTSAN_LIB_PATH, LD_PRELOAD=rt,
+  # the sanitizer runtime goes in front of whatever the environment already preloads (it must come first)
+  preload = ':'.join(p for p in (rt, os.environ.get('LD_PRELOAD', '')) if p)
+  env = dict(os.environ, TMX_LIB=tb.HOSTSAN_LIB_PATH, LD_PRELOAD=preload,
              ASAN_OPTIONS='detect_leaks=0:abort_on_error=1', UBSAN_OPTIONS='halt_on_error=1:print_stacktrace=1')
   child = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'host_sanitizer_child.py')
   res = subprocess.run([sys.executable, child], capture_output=True, text=True, env=env, timeout=300)
