@@ -1802,20 +1802,22 @@ static int slice_len(int KT, int s) { return ((KT + s - 1) / s + 3) / 4 * 4; }
 static bool slices_ok(int KT, int s) { return (KT + slice_len(KT, s) - 1) / slice_len(KT, s) == s; }
 
 // Number of K-slices for a projection: the count that minimises (rounds of workgroups over the
-// 256 CUs) x (steps per slice + fixed start-up / reduction work), with a small charge per plane
-// for the f32 traffic of the partial sums.  No slice may be empty.
-// Number of K-slices for a projection.  Wide projections (>= 192 column blocks) are not
-// split: they write bf16 directly.  Otherwise the smallest power of two that gives at least
-// 128 workgroups and at most 32 k-tiles per slice, in whole groups of 4 k-tiles, no empty slice.
+// device's CUs: 256 on the MI355X, also assumed when no device is present) x (steps per slice + fixed
+// start-up / reduction work), with a small charge per plane for the f32 traffic of the partial sums.
+// No slice may be empty.
+// The four-wave kernel: wide projections (column blocks for three quarters of the CUs) are not
+// split: they write bf16 directly.  Otherwise the smallest power of two that gives workgroups for
+// half of the CUs and at most 32 k-tiles per slice, in whole groups of 4 k-tiles, no empty slice.
 static int num_splits4(int K, int N) {
   const int nblocks = (N + 127) / 128;
   const int KT = K / 64;
-  if (nblocks >= 192) return 1;
+  const int cus = device_cus();
+  if (nblocks >= cus * 3 / 4) return 1;
   int best = 1;
   for (int s = 1; s <= TMX_MAX_SPLITS; s *= 2) {
     if (!slices_ok(KT, s)) break;
     best = s;
-    if (nblocks * s >= 128 && slice_len(KT, s) <= 32) break;
+    if (nblocks * s >= cus / 2 && slice_len(KT, s) <= 32) break;
   }
   return best;
 }
@@ -1826,7 +1828,7 @@ int qlinear_num_splits(int K, int N, int M) {
     // 256-row blocks: K-slices only while the launch has fewer workgroups than CUs
     const int wgs = (N + 255) / 256 * ((M + 255) / 256);
     int s = 1;
-    while (wgs * s < 192 && s * 2 <= TMX_MAX_SPLITS && slices_ok(K / 64, s * 2) && slice_len(K / 64, s * 2) >= 8) s *= 2;
+    while (wgs * s < device_cus() * 3 / 4 && s * 2 <= TMX_MAX_SPLITS && slices_ok(K / 64, s * 2) && slice_len(K / 64, s * 2) >= 8) s *= 2;
     return s;
   }
   if (four_wave(K, N)) return num_splits4(K, N);
@@ -1838,11 +1840,12 @@ int qlinear_num_splits(int K, int N, int M) {
   // charge per plane covers the consumer's reads (measured on the o projection: 4 slices beat 6)
   const int ks = (M > 64 || K % 256 == 0) ? 4 : 8;
   const int nls = qlinear_num_lora_splits(K, N);
+  const int cus = device_cus();
   int best = 1;
   float best_cost = 1e30f;
   for (int s = 1; s <= TMX_MAX_SPLITS; ++s) {
     if (!slices_ok(KT, s)) continue;
-    const int rounds = (nblocks * s + (nls + s - 1) / s * s + 255) / 256;
+    const int rounds = (nblocks * s + (nls + s - 1) / s * s + cus - 1) / cus;
     const int nsteps = (slice_len(KT, s) + ks - 1) / ks;
     const float cost = rounds * (nsteps + (ks == 4 ? 4.0f : 2.0f)) + (ks == 4 ? 0.6f : 0.15f) * s;
     if (cost < best_cost) { best_cost = cost; best = s; }
