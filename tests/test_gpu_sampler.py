@@ -74,6 +74,30 @@ def test_toy_config_greedy_matches_oracle():
   _compare_greedy(out, ref, 4, 40)
 
 
+def test_streaming_copy_of_the_head_changes_nothing():
+  """A rollout whose steps stream the head from its tile copy (the default) against one that reads the row-major
+  matrix: tokens and log-probs are identical bit for bit, greedy and sampled (tied and untied heads)."""
+  for tied in (False, True):
+    cfg = OM.Config('llama3', 2, 1024, 256, 512, 4, 64, 2, rope_theta=10000, norm_eps=1e-5, tied=tied)
+    rng = np.random.default_rng(3)
+    prompts = [rng.integers(3, cfg.vocab_size, n) for n in (9, 14, 5)]
+    outs = []
+    for stream_head in (True, False):
+      _, model = _pair(cfg, seed=41)
+      model.stream_head = stream_head
+      s = _sampler(model, cfg, 48)
+      greedy = s(prompt_token_ids=prompts, max_generation_steps=12, return_logprobs=True, eos_tokens=[-1])
+      sampled = s(prompt_token_ids=prompts, max_generation_steps=12, return_logprobs=True, eos_tokens=[-1],
+                  temperature=0.8, top_p=1.0, seed=7)
+      assert (model.desc().head_tiles is not None) == stream_head
+      outs.append((greedy, sampled))
+    for a, b in zip(outs[0], outs[1]):
+      for ta, tb in zip(a.tokens, b.tokens):
+        np.testing.assert_array_equal(ta, tb)
+      for la, lb in zip(a.logprobs, b.logprobs):
+        np.testing.assert_array_equal(np.asarray(la), np.asarray(lb))
+
+
 def test_wide_layer_with_the_projection_side_lora_delta_matches_oracle():
   """One layer at the 8B width (d 4096, SwiGLU 14336, 32 / 8 heads of 128), LoRA r16 on every projection,
   6 sequences: the down projection is long enough (7 K-slices of 2048) for its own launch to finish the
