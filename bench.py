@@ -539,8 +539,27 @@ def main():
     sampler.check_device_status(st)
     result['prompt_kv_sharing']['attention_ms_per_step'] = tot / n_prof
     result['prompt_kv_sharing']['attention_ms_per_step_without'] = result['kernel_ms_per_step']['attention']
+  if args.steps + args.warmup >= new and not args.sync_steps:
+    # The whole rollout through the call a user makes (Sampler.__call__): padding, cache fill over the prompt,
+    # every decode step, the device status check, device-to-host copies and per-row slicing.  Beside `value`,
+    # which times decode steps alone.
+    sampler.share_prompt_kv = not args.no_kv_sharing
+    prompts = [row for row in ids]
+    best = None
+    for rep in range(2):
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      out = sampler(prompt_token_ids=prompts, max_generation_steps=new, return_logprobs=True, eos_tokens=[-1],
+                    temperature=temp, top_p=top_p, seed=rep)
+      torch.cuda.synchronize()
+      sec = time.perf_counter() - t0
+      n_tok = int(sum(len(t) for t in out.tokens))
+      assert n_tok == batch * new
+      best = sec if best is None else min(best, sec)
+    result['sampler_call'] = {'tokens_per_s': n_tok / best, 'seconds': best, 'generated_tokens': n_tok,
+                              'includes': 'prompt padding, cache fill, decode steps, status check, copies to the host'}
   if not args.no_cpu_baseline and not cfg.num_experts:
-    del st
+    st = None
     result['cpu_baseline'] = cpu_baseline(args.workload)
   print(json.dumps(result))
 
