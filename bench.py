@@ -427,8 +427,14 @@ def main():
       symbols = {'tmx::sb_linear_kernel<1, 0>': ['qkv_linear'], 'tmx::sb_linear_kernel<2, 1>': ['o_linear'],
                  'tmx::sb_linear_kernel<1, 2>': ['gate_up_linear'], 'tmx::sb_linear_kernel<0, 1>': ['down_linear'],
                  f'tmx::sb_attn_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention']}
+    # the walk of the run without shared slots: on the matrix pipe for 4 or 8 query heads per kv head while three
+    # workgroups per CU hold every (sequence, kv head) pair at once (+ gqa_combine_kernel where a row is split),
+    # else on the vector ALU
+    g_heads = cfg.num_heads // cfg.num_kv_heads
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    on_tile = g_heads in (4, 8) and batch * cfg.num_kv_heads <= 3 * cus
     symbols.update({} if small else {
-        f'tmx::gqa_decode_kernel<{cfg.head_dim}, {cfg.num_heads // cfg.num_kv_heads}>': ['attention']})
+        f"tmx::gqa_{'tile' if on_tile else 'decode'}_kernel<{cfg.head_dim}, {g_heads}>": ['attention']})
     symbols.update({
         # more than 64 rows: the head in 256 x 256 blocks (template argument: the sampling mode, 1 = top-p branch);
         # with top_p < 1 the class also holds the three selection launches of nucleus.hip

@@ -226,11 +226,12 @@ __global__ __launch_bounds__(H) void gqa_combine_kernel(AttnArgs a) {
 // MFMA tile: scores^T [position, query] = K . Q^T and out^T [hidden, query] += V^T . P^T as in the many-tokens
 // kernel below, with the four waves of a workgroup taking different blocks of 32 positions and meeting through
 // LDS at the end.  K rows go from global memory straight into the A operand (lane (position, h) owns one half
-// of its row), the V tile of a wave goes global -> LDS by direct loads and is gathered transposed with 16-bit
-// reads, the query fragments wait in LDS.  Per 32 positions a wave issues 8 + 32 MFMAs and about 150 VALU
-// instructions, against about 1400 VALU instructions per 16 positions of gqa_decode_walk, whose dot products
-// and reductions run on the vector ALU; it takes the launch wherever its workgroups (three per CU: LDS and
-// registers) are all resident at once.
+// of its row), the V tile of a wave goes global -> LDS by direct loads and is read transposed
+// (ds_read_b64_tr_b16: 16 reads per 32 positions where 16-bit gathers took 64 reads and 32 merges), the query
+// fragments wait in LDS.  Per 32 positions a wave issues 8 + 32 MFMAs and about 120 VALU instructions, against
+// 527 VALU instructions per 16 positions of gqa_decode_walk at 4 query heads (about 1400 at 8), whose dot
+// products and reductions run on the vector ALU; it takes the launch wherever its workgroups (three per CU:
+// LDS and registers) are all resident at once.
 //
 // Two kinds of query block share the launch:
 //  * a row: the G query heads of one sequence (the first G columns of the tile) over that sequence's own slots;
@@ -380,31 +381,36 @@ __device__ __forceinline__ void gqa_tile_walk(const AttnArgs& a, PrefixLds<H>& l
         for (int r = 0; r < 16; ++r) o[c][r] *= alpha;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this block's V tile has landed
-    // out^T += V^T . P^T, 16 positions (accumulator registers 8 kb .. 8 kb + 7) per MFMA.  The V^T fragment is
-    // gathered with 16-bit reads: element (row, hidden 32 c + qi) of the tile, row = acc_row(8 kb + j, lane) =
-    // 8 (2 kb + j / 4) + 4 h + j % 4, sits in chunk (4 c + qi / 8) ^ row % CPR; the lane's share of that XOR is
-    // one word (gsw), the rest a constant per read, and the addresses are formed here, read by read
+    // out^T += V^T . P^T, 16 positions (accumulator registers 8 kb .. 8 kb + 7) per MFMA.  The V^T fragment of
+    // lane (hidden 32 c + qi, h) is positions acc_row(8 kb + j, lane) = 16 kb + 8 (j / 4) + 4 h + j % 4, j = 0..7:
+    // two runs of four consecutive rows of one column of the tile, which the transposing LDS read delivers
+    // directly (ds_read_b64_tr_b16: in every 16 lanes, lane 4 k + q supplies the address of four consecutive
+    // 16-bit elements M[4 k + q][0..3] and lane 4 q' + c' receives M[4 k + q'][c'], k = 0..3).  So lane
+    // (k4, q4) of a group points at row run + 4 h + k4, columns 32 c + 16 (group % 2) + 4 q4 .. + 3, and a read
+    // returns the four rows of the lane's own column.  Chunk (column / 8) of row r sits at chunk ^ r % CPR; the
+    // lane's share of that XOR is one word (lsw), the rest a constant per read.
     {
-      int gsw = (qi >> 3) ^ ((4 * h) % CPR), gbase = 4 * h * H + (qi & 7);
-      asm volatile("" : "+v"(gsw), "+v"(gbase));
+      const int k4 = (lane & 15) >> 2, q4 = lane & 3, g2 = (lane >> 4) & 1;
+      int lsw = (2 * g2 + (q4 >> 1)) ^ (4 * h + k4), lbase = (4 * h + k4) * H + 4 * (q4 & 1);
+      asm volatile("" : "+v"(lsw), "+v"(lbase));
+      typedef short s16x4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
       for (int kb2 = 0; kb2 < 2; ++kb2) {
         const u32x4_t pf = {pk[4 * kb2], pk[4 * kb2 + 1], pk[4 * kb2 + 2], pk[4 * kb2 + 3]};
         const u32x4_t pg = {pl2[4 * kb2], pl2[4 * kb2 + 1], pl2[4 * kb2 + 2], pl2[4 * kb2 + 3]};
 #pragma unroll
         for (int c = 0; c < HT; ++c) {
-          uint32_t vw[4];
+          s16x4_t run[2];
 #pragma unroll
-          for (int j2 = 0; j2 < 4; ++j2) {
-            uint32_t e2[2];
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-              const int j = 2 * j2 + e;
-              const int row0 = (2 * kb2 + j / 4) * 8 + (j & 3);  // the row without the lane's 4 h
-              e2[e] = vt[gbase + row0 * H + ((gsw ^ (4 * c) ^ (row0 % CPR)) << 3)];
-            }
-            vw[j2] = e2[0] | (e2[1] << 16);
+          for (int a2 = 0; a2 < 2; ++a2) {
+            const int row0 = 16 * kb2 + 8 * a2;  // the run without the lane's 4 h + k4
+            const uint16_t* src = vt + lbase + row0 * H + ((lsw ^ (4 * c) ^ (row0 % CPR)) << 3);
+            run[a2] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4_t*)(src));
           }
+          uint32_t vw[4];
+          __builtin_memcpy(&vw[0], &run[0], 8);
+          __builtin_memcpy(&vw[2], &run[1], 8);
           const u32x4_t vf = {vw[0], vw[1], vw[2], vw[3]};
           o[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
                                                          __builtin_bit_cast(bf16x8_t, pf), o[c], 0, 0, 0);
@@ -563,7 +569,7 @@ __global__ __launch_bounds__(256, 3) void gqa_shared_kernel(AttnArgs a, int n_gr
 //     accumulator, so mask, max, exp and sum run down the registers (one shuffle joins the halves);
 //   out^T [hidden, query] += V^T . P^T  : the B operand is the lane's own 8 probabilities of a
 //     16-position block (positions are consumed in accumulator order, which V^T follows: its
-//     fragment is gathered from the V tile with 16-bit LDS reads), and the rescale by
+//     fragment comes from the V tile by transposing LDS reads), and the rescale by
 //     exp(old max - new max) is per lane.
 // Probabilities enter the product as two bf16 terms (hi + lo), i.e. with 16 mantissa bits.
 constexpr int kFillMinTokens = 4;  // tokens per sequence and pass from which the fill kernel is used
@@ -682,19 +688,22 @@ __global__ __launch_bounds__(256) void gqa_fill_kernel(AttnArgs a) {
       const u32x4_t pg = {pl2[4 * kb2], pl2[4 * kb2 + 1], pl2[4 * kb2 + 2], pl2[4 * kb2 + 3]};
 #pragma unroll
       for (int c = 0; c < HT; ++c) {
-        uint32_t vw[4];
+        // V^T fragment: two runs of four consecutive rows of the lane's column, by the transposing LDS read
+        // (see gqa_tile_walk): lane (k4, q4) of a group of 16 points at row run + 4 h + k4, columns
+        // 32 c + 16 (group % 2) + 4 q4 .. + 3
+        typedef short s16x4_t __attribute__((ext_vector_type(4)));
+        const int k4 = (lane & 15) >> 2, q4 = lane & 3, g2 = (lane >> 4) & 1;
+        s16x4_t run[2];
 #pragma unroll
-        for (int j2 = 0; j2 < 4; ++j2) {
-          uint32_t e2[2];
-#pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            const int j = 2 * j2 + e;
-            const int row = (2 * kb2 + j / 4) * 8 + 4 * h + (j & 3);  // = acc_row(8 kb2 + j, lane)
-            const int chunk = 4 * c + (qi >> 3);
-            e2[e] = vt[buf][row * H + ((chunk ^ (row % CPR)) * 8) + (qi & 7)];
-          }
-          vw[j2] = e2[0] | (e2[1] << 16);
+        for (int a2 = 0; a2 < 2; ++a2) {
+          const int row = 16 * kb2 + 8 * a2 + 4 * h + k4;
+          const int chunk = 4 * c + 2 * g2 + (q4 >> 1);
+          run[a2] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(
+              &vt[buf][row * H + ((chunk ^ (row % CPR)) * 8) + 4 * (q4 & 1)]));
         }
+        uint32_t vw[4];
+        __builtin_memcpy(&vw[0], &run[0], 8);
+        __builtin_memcpy(&vw[2], &run[1], 8);
         const u32x4_t vf = {vw[0], vw[1], vw[2], vw[3]};
         o[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
                                                        __builtin_bit_cast(bf16x8_t, pf), o[c], 0, 0, 0);
@@ -781,8 +790,12 @@ static AttnPlan plan_attention(int B, int N, int Kh, int H, int C, int share_gs,
   p.shared = attn_share_ok(B, N, Kh, H, C, share_gs, share_len);
   // Rows' own slots: the tile walk for 8 query heads per kv head (measured on the 30B-A3B shape, 32 sequences at
   // context 512: 10.7 + 3.0 us for walk and combine against 21.7 + 3.9 us; the vector walk's work per cache row
-  // grows with the heads); up to 4 heads the vector walk (see gqa_shared_kernel).
+  // grows with the heads); up to 2 heads, and 4 heads behind shared slots, the vector walk (see gqa_shared_kernel).
   p.tile = G == 8 && pairs <= (p.shared ? 2 * slots : slots);
+  // 4 heads per kv head without shared slots: the tile walk as well, since its V^T fragments come from the
+  // transposing LDS read (measured on the 8B shape, 64 sequences, whole rollout: 4.158 -> 4.109 ms per step; with
+  // shared slots the rows stay on the vector walk: 3.941 against 3.953)
+  if (G == 4 && !p.shared && pairs <= slots) p.tile = true;
   if (G == 8 && !p.tile) p.shared = false;
   if (p.shared && pairs > 2 * slots) p.shared = false;
   long group_wgs = 0;
