@@ -64,6 +64,9 @@ extern "C" {
                               :207-226 selective_log_softmax) */
 
 const char* tmx_status_string(int status);
+/* Bumped whenever a struct of this header grows or an entry point changes: 7 = tmx_model_desc.head_tiles and the
+ * tmx_decode_state.share_* fields are present.  A caller that fills the structs checks it once after loading. */
+#define TMX_ABI_VERSION 7
 int tmx_abi_version(void);
 
 /* w_out[K, N] bf16 = bf16(q) * scale evaluated in bf16, bit-exact.

@@ -51,7 +51,9 @@ def test_header_is_plain_c_and_cxx():
 
 def test_status_strings_and_version():
   lib = _lib.lib()
-  assert lib.tmx_abi_version() == 7
+  assert lib.tmx_abi_version() == 7 == _lib.ABI_VERSION
+  header = open(os.path.join(os.path.dirname(os.path.abspath(__file__)), '..', 'include', 'tmx.h')).read()
+  assert '#define TMX_ABI_VERSION 7' in header
   assert lib.tmx_status_string(0) == b'ok'
   for code in (-1, -2, -3, -4):
     assert len(lib.tmx_status_string(code)) > 5

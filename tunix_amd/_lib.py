@@ -9,6 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('TMX_LIB', os.path.join(_HERE, 'libtmx.so'))
 
 _lib = None
+ABI_VERSION = 7  # TMX_ABI_VERSION of include/tmx.h
 
 vp, ci, cf, cu32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_uint32
 
@@ -85,6 +86,11 @@ def lib():
       fn.restype = ctypes.c_size_t
     l.tmx_status_string.argtypes = [ci]
     l.tmx_status_string.restype = ctypes.c_char_p
+    # the ctypes structs of model.py mirror the header of ABI_VERSION: a library built from another header
+    # would read them with the wrong layout
+    if l.tmx_abi_version() != ABI_VERSION:
+      raise TmxError(f'{LIB_PATH} has ABI version {l.tmx_abi_version()}, this package expects {ABI_VERSION}: '
+                     'rebuild it with `python -m tunix_amd.build`.')
     _lib = l
   return _lib
 

@@ -41,4 +41,4 @@ extern "C" const char* tmx_status_string(int status) {
   }
 }
 
-extern "C" int tmx_abi_version(void) { return 7; }
+extern "C" int tmx_abi_version(void) { return TMX_ABI_VERSION; }
